@@ -1,0 +1,116 @@
+// Variant registry, dispatcher and harness helpers of the C ABI (include/hgemm.h).
+#include "../../include/hgemm.h"
+#include "common.h"
+#include "variant_def.h"
+
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_base);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_padding);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_swizzle);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_pg2s);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_pg2s_ps2r);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_stage2);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_stage3);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_stage4);
+HGEMM_DECLARE_SUPPORTS(hgemm_skinny);
+HGEMM_DECLARE_SUPPORTS(hgemm_auto);
+
+namespace {
+
+int any_shape(size_t M, size_t N, size_t K) { return M > 0 && N > 0 && K > 0; }
+int naive_mfma_shape(size_t M, size_t N, size_t K) {
+    return M > 0 && N > 0 && K > 0 && M % 32 == 0 && N % 32 == 0 && K % 16 == 0;
+}
+
+struct Variant {
+    const char *name;    // display name, as in the reference's evaluate() calls (src/main.cu:100-123)
+    const char *symbol;  // exported function
+    hgemm_fn fn;
+    int (*supports)(size_t, size_t, size_t);
+    int in_default_run;  // the reference comments the naive / base kernels out of its run
+};
+
+const Variant kVariants[] = {
+    {"Simt-Naive", "hgemm_simt_naive", hgemm_simt_naive, any_shape, 0},
+    {"Mfma-Naive", "hgemm_mfma_naive", hgemm_mfma_naive, naive_mfma_shape, 0},
+    {"Mfma-Base", "hgemm_mfma_base", hgemm_mfma_base, hgemm_mfma_base_supports, 0},
+    {"Mfma-Padding", "hgemm_mfma_padding", hgemm_mfma_padding, hgemm_mfma_padding_supports, 1},
+    {"Mfma-Swizzle", "hgemm_mfma_swizzle", hgemm_mfma_swizzle, hgemm_mfma_swizzle_supports, 1},
+    {"Mfma-Async", "hgemm_mfma_async", hgemm_mfma_async, hgemm_mfma_async_supports, 1},
+    {"Mfma-Async-Pg2s", "hgemm_mfma_async_pg2s", hgemm_mfma_async_pg2s, hgemm_mfma_async_pg2s_supports, 1},
+    {"Mfma-Async-Pg2s-Ps2r", "hgemm_mfma_async_pg2s_ps2r", hgemm_mfma_async_pg2s_ps2r,
+     hgemm_mfma_async_pg2s_ps2r_supports, 1},
+    {"Mfma-Async-Stage2", "hgemm_mfma_async_stage2", hgemm_mfma_async_stage2, hgemm_mfma_async_stage2_supports, 1},
+    {"Mfma-Async-Stage3", "hgemm_mfma_async_stage3", hgemm_mfma_async_stage3, hgemm_mfma_async_stage3_supports, 1},
+    {"Mfma-Async-Stage4", "hgemm_mfma_async_stage4", hgemm_mfma_async_stage4, hgemm_mfma_async_stage4_supports, 1},
+    {"Skinny", "hgemm_skinny", hgemm_skinny, hgemm_skinny_supports, 1},
+    {"Auto", "hgemm_auto", hgemm_auto, hgemm_auto_supports, 1},
+};
+constexpr int kVariantCount = (int)(sizeof(kVariants) / sizeof(kVariants[0]));
+
+const Variant *variant_at(int index) {
+    HGEMM_CHECK_MSG(index >= 0 && index < kVariantCount, "variant index %d out of range [0, %d)", index,
+                    kVariantCount);
+    return &kVariants[index];
+}
+
+}  // namespace
+
+extern "C" int hgemm_variant_count(void) { return kVariantCount; }
+extern "C" const char *hgemm_variant_name(int index) { return variant_at(index)->name; }
+extern "C" const char *hgemm_variant_symbol(int index) { return variant_at(index)->symbol; }
+extern "C" hgemm_fn hgemm_variant_fn(int index) { return variant_at(index)->fn; }
+extern "C" int hgemm_variant_in_default_run(int index) { return variant_at(index)->in_default_run; }
+
+extern "C" int hgemm_variant_find(const char *name) {
+    if (!name) return -1;
+    for (int i = 0; i < kVariantCount; ++i)
+        if (strcmp(name, kVariants[i].name) == 0 || strcmp(name, kVariants[i].symbol) == 0) return i;
+    return -1;
+}
+
+extern "C" int hgemm_variant_supports(int index, size_t M, size_t N, size_t K) {
+    if (M == 0 || N == 0 || K == 0) return 0;
+    if (M * K >= (1ull << 31) || N * K >= (1ull << 31) || M * N >= (1ull << 31)) return 0;
+    return variant_at(index)->supports(M, N, K);
+}
+
+// Timing loop of Tester::profile (reference src/common/tester.h:89-97) with the event
+// handling of CudaTimer (reference src/common/cuda_timer.h:32-42): events on the null
+// stream, no synchronisation between the timed calls.
+extern "C" double hgemm_profile_ms(hgemm_fn fn, const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M,
+                                   size_t N, size_t K, size_t warmup, size_t iterations) {
+    const hgemm_half *As[1] = {A};
+    const hgemm_half *Bs[1] = {B};
+    hgemm_half *Cs[1] = {C};
+    return hgemm_profile_rotating_ms(fn, As, Bs, Cs, 1, M, N, K, warmup, iterations);
+}
+
+extern "C" double hgemm_profile_rotating_ms(hgemm_fn fn, const hgemm_half *const *A, const hgemm_half *const *B,
+                                            hgemm_half *const *C, size_t n_sets, size_t M, size_t N, size_t K,
+                                            size_t warmup, size_t iterations) {
+    HGEMM_CHECK(fn != nullptr);
+    HGEMM_CHECK_GT(n_sets, 0u);
+    HGEMM_CHECK_GT(iterations, 0u);
+    hipEvent_t start = nullptr, stop = nullptr;
+    HGEMM_CHECK_HIP_ERROR(hipEventCreate(&start));
+    HGEMM_CHECK_HIP_ERROR(hipEventCreate(&stop));
+    for (size_t i = 0; i < warmup; ++i) fn(A[i % n_sets], B[i % n_sets], C[i % n_sets], M, N, K);
+    HGEMM_CHECK_HIP_ERROR(hipEventRecord(start, nullptr));
+    for (size_t i = 0; i < iterations; ++i) fn(A[i % n_sets], B[i % n_sets], C[i % n_sets], M, N, K);
+    HGEMM_CHECK_HIP_ERROR(hipEventRecord(stop, nullptr));
+    HGEMM_CHECK_HIP_ERROR(hipEventSynchronize(stop));
+    float ms = 0.0f;
+    HGEMM_CHECK_HIP_ERROR(hipEventElapsedTime(&ms, start, stop));
+    HGEMM_CHECK_HIP_ERROR(hipEventDestroy(start));
+    HGEMM_CHECK_HIP_ERROR(hipEventDestroy(stop));
+    return (double)ms / (double)iterations;
+}
+
+extern "C" double hgemm_tflops(size_t M, size_t N, size_t K, double ms) {
+    return (double)(M * N * K * 2) * 1e-12 / (ms * 1e-3);
+}
+
+extern "C" double hgemm_bytes(size_t M, size_t N, size_t K) { return 2.0 * ((double)M * K + (double)K * N + (double)M * N); }
+
+extern "C" const char *hgemm_version(void) { return "hgemm-gfx950 0.1"; }

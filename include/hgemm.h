@@ -1,0 +1,131 @@
+/*
+ * hgemm.h -- C ABI of the MI355X (gfx950) half-precision GEMM library.
+ *
+ * Every kernel entry point has the shape of the reference's HGEMM_FUNC
+ * (reference src/main.cu:11):
+ *
+ *     void name(half *A, half *B, half *C, size_t M, size_t N, size_t K)
+ *
+ * and computes  C[m*N + n] = sum_k A[m*K + k] * B[n*K + k]  (reference
+ * src/simt_naive.cu:18-24) on DEVICE pointers the caller owns:
+ *     A  row-major   M x K                      (reference src/common/tester.h:117)
+ *     B  column-major K x N, i.e. N rows of K    (reference src/common/tester.h:118)
+ *     C  row-major   M x N, fully overwritten    (reference src/common/tester.h:119)
+ * Elements are IEEE binary16 (2 bytes).  Products are accumulated in fp32 and rounded to
+ * fp16 once (the reference accumulates in fp16; this is the one deliberate difference).
+ *
+ * Calling convention, as in the reference (src/mma/mma_async_stage4.cu:637-644,
+ * src/common/tester.h:59-62,91-94): launched asynchronously on the null stream, nothing is
+ * allocated per call, the caller synchronises.  A contract violation (null pointer, zero
+ * dimension, a shape the variant cannot tile) is reported on stderr and ends the process
+ * with EXIT_FAILURE, the convention of the reference's HGEMM_CHECK macros
+ * (src/common/common.h:23-29); unlike the reference, unsupported shapes are diagnosed
+ * instead of being read out of bounds.  hgemm_variant_supports() lets a caller ask first.
+ */
+#ifndef HGEMM_H_
+#define HGEMM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* 16-bit storage type of one element; bit-compatible with _Float16 / __half. */
+typedef uint16_t hgemm_half;
+
+typedef void (*hgemm_fn)(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K);
+
+#define HGEMM_FUNC(name) \
+    void name(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K)
+
+/* One thread per output element, fp32 accumulate; any shape.
+ * Replaces simtNaive (reference src/simt_naive.cu:27). */
+HGEMM_FUNC(hgemm_simt_naive);
+
+/* One wavefront per 32x32 tile of C straight from global memory on
+ * v_mfma_f32_32x32x16_f16; needs M%32 == N%32 == 0, K%16 == 0.
+ * Replaces wmmaNaive / mmaNaive (reference src/wmma/wmma_naive.cu:46, src/mma/mma_naive.cu:70). */
+HGEMM_FUNC(hgemm_mfma_naive);
+
+/* Block-tiled ladder.  Each step adds one technique to the previous one, the way the
+ * reference's files do.  Shape needs are those of the tile (see hgemm_variant_supports). */
+/* LDS-staged 256x128x32 tile, plain row-major LDS rows.
+ * Replaces wmmaBase / mmaBase (reference src/wmma/wmma_base.cu:194, src/mma/mma_base.cu:200). */
+HGEMM_FUNC(hgemm_mfma_base);
+/* + 16-byte row padding against LDS bank conflicts.
+ * Replaces wmmaPadding (reference src/wmma/wmma_padding.cu:196). */
+HGEMM_FUNC(hgemm_mfma_padding);
+/* + XOR-swizzled LDS rows instead of padding.
+ * Replaces mmaPermuted (reference src/mma/mma_permuted.cu:224). */
+HGEMM_FUNC(hgemm_mfma_swizzle);
+/* + global -> LDS copies that bypass registers (global_load_lds_dwordx4).
+ * Replaces wmmaAsync / mmaAsync (reference src/wmma/wmma_async.cu:207, src/mma/mma_async.cu:233). */
+HGEMM_FUNC(hgemm_mfma_async);
+/* + two LDS buffers: the next K chunk is fetched while the current one is multiplied.
+ * Replaces wmmaAsyncPg2s / mmaAsyncPg2s (reference src/wmma/wmma_async_pg2s.cu:282,
+ * src/mma/mma_async_pg2s.cu:323). */
+HGEMM_FUNC(hgemm_mfma_async_pg2s);
+/* + double-buffered MFMA operand registers (LDS -> register prefetch).
+ * Replaces wmmaAsyncPg2sPs2r / mmaAsyncPg2sPs2r (reference src/wmma/wmma_async_pg2s_ps2r.cu:346,
+ * src/mma/mma_async_pg2s_ps2r.cu:412). */
+HGEMM_FUNC(hgemm_mfma_async_pg2s_ps2r);
+/* K_STAGE-deep LDS ring, s_waitcnt vmcnt(n) in place of cp.async.wait_group.
+ * Replace wmmaAsyncStage2/3 and mmaAsyncStage2/3/4 (reference src/wmma/wmma_async_stage2.cu:375,
+ * src/wmma/wmma_async_stage3.cu:453, src/mma/mma_async_stage2.cu:447,
+ * src/mma/mma_async_stage3.cu:542, src/mma/mma_async_stage4.cu:637). */
+HGEMM_FUNC(hgemm_mfma_async_stage2);
+HGEMM_FUNC(hgemm_mfma_async_stage3);
+HGEMM_FUNC(hgemm_mfma_async_stage4);
+
+/* Small-M (decode-shaped) product: streams B once, bound by HBM bandwidth, M <= 128.
+ * No counterpart in the reference, whose tiled kernels cannot run M < 256
+ * (reference src/mma/mma_async_stage4.cu:64-66,93-94). */
+HGEMM_FUNC(hgemm_skinny);
+
+/* Dispatcher: picks the tile / kernel for the shape; accepts every shape with
+ * K % 8 == 0 through the MFMA kernels and anything else through the scalar kernel.
+ * This is the entry point the benchmark measures. */
+HGEMM_FUNC(hgemm_auto);
+
+/* ---- registry, so a driver can enumerate variants the way the reference's main lists
+ * them (reference src/main.cu:100-123) without an edit per variant. ---- */
+int hgemm_variant_count(void);
+/* Display name used in the log line, e.g. "Mfma-Async-Stage4" (reference src/main.cu:120). */
+const char *hgemm_variant_name(int index);
+/* Exported symbol name, e.g. "hgemm_mfma_async_stage4". */
+const char *hgemm_variant_symbol(int index);
+hgemm_fn hgemm_variant_fn(int index);
+/* Index of a variant by display or symbol name, -1 if unknown. */
+int hgemm_variant_find(const char *name);
+/* 1 if variant `index` can run the shape, 0 otherwise (no side effects). */
+int hgemm_variant_supports(int index, size_t M, size_t N, size_t K);
+/* 1 if the variant belongs to the default run (reference src/main.cu:100-123 comments the
+ * slow ones out), 0 otherwise. */
+int hgemm_variant_in_default_run(int index);
+
+/* ---- harness helpers: the timing loop of Tester::profile with CudaTimer semantics
+ * (reference src/common/tester.h:89-97, src/common/cuda_timer.h:32-42). ---- */
+/* Runs `warmup` untimed calls, then `iterations` back-to-back calls bracketed by a pair of
+ * HIP events on the null stream; returns the average milliseconds per call. */
+double hgemm_profile_ms(hgemm_fn fn, const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N,
+                        size_t K, size_t warmup, size_t iterations);
+/* As above, but call i uses operand set i % n_sets (A[i], B[i], C[i]) so that repeated
+ * calls on small operands stream from HBM instead of the on-chip caches. */
+double hgemm_profile_rotating_ms(hgemm_fn fn, const hgemm_half *const *A, const hgemm_half *const *B,
+                                 hgemm_half *const *C, size_t n_sets, size_t M, size_t N, size_t K, size_t warmup,
+                                 size_t iterations);
+/* 2*M*N*K*1e-12 / (ms*1e-3)  (reference src/common/tester.h:96-97). */
+double hgemm_tflops(size_t M, size_t N, size_t K, double ms);
+/* Algorithmic bytes of one call: 2*(M*K + K*N + M*N). */
+double hgemm_bytes(size_t M, size_t N, size_t K);
+
+/* Library version string. */
+const char *hgemm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* HGEMM_H_ */
