@@ -1,0 +1,209 @@
+"""ctypes binding of ``include/hgemm.h`` / ``include/hgemm_hipblaslt.h``.
+
+Operand layouts are the reference's (``src/common/tester.h:117-120``): ``A`` is ``(M, K)``
+row-major, ``B`` is handed over as its ``(N, K)`` storage (column-major ``K x N``), ``C`` is
+``(M, N)`` row-major; all fp16, all on the GPU.  Calls are asynchronous on the null stream,
+which is also torch's default stream.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import List, Optional
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def lib_path() -> str:
+    return os.path.join(_HERE, "lib", "libhgemm.so")
+
+
+def vendor_lib_path() -> str:
+    return os.path.join(_HERE, "lib", "libhgemm_hipblaslt.so")
+
+
+def driver_path() -> str:
+    return os.path.join(_HERE, "bin", "hgemm")
+
+
+_SZ = C.c_size_t
+_PTR = C.c_void_p
+_HGEMM_ARGS = [_PTR, _PTR, _PTR, _SZ, _SZ, _SZ]
+HGEMM_FN = C.CFUNCTYPE(None, *_HGEMM_ARGS)
+
+# every symbol include/hgemm.h declares
+KERNEL_SYMBOLS = [
+    "hgemm_simt_naive", "hgemm_mfma_naive", "hgemm_mfma_base", "hgemm_mfma_padding", "hgemm_mfma_swizzle",
+    "hgemm_mfma_async", "hgemm_mfma_async_pg2s", "hgemm_mfma_async_pg2s_ps2r", "hgemm_mfma_async_stage2",
+    "hgemm_mfma_async_stage3", "hgemm_mfma_async_stage4", "hgemm_skinny", "hgemm_auto",
+]
+HELPER_SYMBOLS = [
+    "hgemm_auto_plan", "hgemm_kernel_name", "hgemm_variant_count", "hgemm_variant_name", "hgemm_variant_symbol",
+    "hgemm_variant_fn", "hgemm_variant_find", "hgemm_variant_supports", "hgemm_variant_in_default_run",
+    "hgemm_profile_ms", "hgemm_profile_rotating_ms", "hgemm_tflops", "hgemm_bytes", "hgemm_version",
+]
+
+
+def _tensor_ptr(t, rows: int, cols: int, what: str) -> int:
+    import torch
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{what}: expected a torch.Tensor, got {type(t).__name__}")
+    if t.dtype != torch.float16:
+        raise TypeError(f"{what}: expected float16, got {t.dtype}")
+    if not t.is_cuda:
+        raise ValueError(f"{what}: must live on the GPU")
+    if tuple(t.shape) != (rows, cols):
+        raise ValueError(f"{what}: expected shape {(rows, cols)}, got {tuple(t.shape)}")
+    if not t.is_contiguous():
+        raise ValueError(f"{what}: must be contiguous")
+    return t.data_ptr()
+
+
+class HgemmLibrary:
+    """``libhgemm.so`` loaded through ctypes; fails loudly when it has not been built."""
+
+    def __init__(self, path: Optional[str] = None):
+        self.path = path or lib_path()
+        if not os.path.exists(self.path):
+            raise FileNotFoundError(
+                f"{self.path} is missing: build it with `python -m cuda_hgemm_amd.build` (needs hipcc); "
+                "there is no non-HIP fallback")
+        self.dll = C.CDLL(self.path)
+        d = self.dll
+        for name in KERNEL_SYMBOLS:
+            fn = getattr(d, name)
+            fn.argtypes, fn.restype = _HGEMM_ARGS, None
+        d.hgemm_auto_plan.argtypes, d.hgemm_auto_plan.restype = [_SZ, _SZ, _SZ, C.POINTER(C.c_int)], C.c_int
+        d.hgemm_kernel_name.argtypes, d.hgemm_kernel_name.restype = [C.c_int], C.c_char_p
+        d.hgemm_variant_count.argtypes, d.hgemm_variant_count.restype = [], C.c_int
+        d.hgemm_variant_name.argtypes, d.hgemm_variant_name.restype = [C.c_int], C.c_char_p
+        d.hgemm_variant_symbol.argtypes, d.hgemm_variant_symbol.restype = [C.c_int], C.c_char_p
+        d.hgemm_variant_fn.argtypes, d.hgemm_variant_fn.restype = [C.c_int], HGEMM_FN
+        d.hgemm_variant_find.argtypes, d.hgemm_variant_find.restype = [C.c_char_p], C.c_int
+        d.hgemm_variant_supports.argtypes, d.hgemm_variant_supports.restype = [C.c_int, _SZ, _SZ, _SZ], C.c_int
+        d.hgemm_variant_in_default_run.argtypes, d.hgemm_variant_in_default_run.restype = [C.c_int], C.c_int
+        d.hgemm_profile_ms.argtypes = [HGEMM_FN, _PTR, _PTR, _PTR, _SZ, _SZ, _SZ, _SZ, _SZ]
+        d.hgemm_profile_ms.restype = C.c_double
+        d.hgemm_profile_rotating_ms.argtypes = [HGEMM_FN, C.POINTER(_PTR), C.POINTER(_PTR), C.POINTER(_PTR), _SZ, _SZ,
+                                                _SZ, _SZ, _SZ, _SZ]
+        d.hgemm_profile_rotating_ms.restype = C.c_double
+        d.hgemm_tflops.argtypes, d.hgemm_tflops.restype = [_SZ, _SZ, _SZ, C.c_double], C.c_double
+        d.hgemm_bytes.argtypes, d.hgemm_bytes.restype = [_SZ, _SZ, _SZ], C.c_double
+        d.hgemm_version.argtypes, d.hgemm_version.restype = [], C.c_char_p
+
+    # ---- registry -------------------------------------------------------------------
+    def variants(self) -> List[dict]:
+        out = []
+        for i in range(self.dll.hgemm_variant_count()):
+            out.append({"index": i, "name": self.dll.hgemm_variant_name(i).decode(),
+                        "symbol": self.dll.hgemm_variant_symbol(i).decode(),
+                        "default_run": bool(self.dll.hgemm_variant_in_default_run(i))})
+        return out
+
+    def find(self, name: str) -> int:
+        idx = self.dll.hgemm_variant_find(name.encode())
+        if idx < 0:
+            raise KeyError(f"unknown hgemm variant {name!r}")
+        return idx
+
+    def supports(self, name: str, M: int, N: int, K: int) -> bool:
+        return bool(self.dll.hgemm_variant_supports(self.find(name), M, N, K))
+
+    def auto_plan(self, M: int, N: int, K: int) -> dict:
+        splits = C.c_int(0)
+        kernel = self.dll.hgemm_auto_plan(M, N, K, C.byref(splits))
+        return {"kernel_id": kernel, "kernel": self.dll.hgemm_kernel_name(kernel).decode(), "splits": splits.value}
+
+    def version(self) -> str:
+        return self.dll.hgemm_version().decode()
+
+    # ---- calls ----------------------------------------------------------------------
+    def fn(self, name: str):
+        """The raw entry point ``void f(const half*, const half*, half*, size_t, size_t, size_t)``."""
+        return getattr(self.dll, self.dll.hgemm_variant_symbol(self.find(name)).decode())
+
+    def call(self, name: str, A, B, C_out, M: int, N: int, K: int) -> None:
+        """Launch variant ``name`` on device tensors; shapes are checked here because the
+        library answers a contract violation by ending the process."""
+        a = _tensor_ptr(A, M, K, "A")
+        b = _tensor_ptr(B, N, K, "B (stored as N rows of K)")
+        c = _tensor_ptr(C_out, M, N, "C")
+        if not self.supports(name, M, N, K):
+            raise ValueError(f"variant {name!r} cannot run M={M} N={N} K={K}")
+        self.fn(name)(a, b, c, M, N, K)
+
+    def profile_ms(self, name: str, A, B, C_out, M: int, N: int, K: int, warmup: int, iterations: int) -> float:
+        """Average milliseconds per call of ``iterations`` back-to-back calls after ``warmup``
+        untimed ones (HIP events on the null stream, the loop of ``Tester::profile``)."""
+        a = _tensor_ptr(A, M, K, "A")
+        b = _tensor_ptr(B, N, K, "B (stored as N rows of K)")
+        c = _tensor_ptr(C_out, M, N, "C")
+        if not self.supports(name, M, N, K):
+            raise ValueError(f"variant {name!r} cannot run M={M} N={N} K={K}")
+        fn = self.dll.hgemm_variant_fn(self.find(name))
+        return self.dll.hgemm_profile_ms(fn, a, b, c, M, N, K, warmup, iterations)
+
+    def profile_fn_rotating_ms(self, fn, As, Bs, Cs, M: int, N: int, K: int, warmup: int, iterations: int) -> float:
+        """Same loop over a cycle of operand sets; ``fn`` is an ``HGEMM_FN`` (ours or the vendor's)."""
+        n = len(As)
+        assert n == len(Bs) == len(Cs) and n > 0
+        pa = (_PTR * n)(*[_tensor_ptr(t, M, K, "A") for t in As])
+        pb = (_PTR * n)(*[_tensor_ptr(t, N, K, "B") for t in Bs])
+        pc = (_PTR * n)(*[_tensor_ptr(t, M, N, "C") for t in Cs])
+        return self.dll.hgemm_profile_rotating_ms(fn, pa, pb, pc, n, M, N, K, warmup, iterations)
+
+    def variant_fn(self, name: str):
+        return self.dll.hgemm_variant_fn(self.find(name))
+
+    def tflops(self, M: int, N: int, K: int, ms: float) -> float:
+        return self.dll.hgemm_tflops(M, N, K, ms)
+
+    def bytes(self, M: int, N: int, K: int) -> float:
+        return self.dll.hgemm_bytes(M, N, K)
+
+
+class VendorLibrary:
+    """``libhgemm_hipblaslt.so``: the hipBLASLt comparator, timed beside the kernels only."""
+
+    def __init__(self, path: Optional[str] = None):
+        self.path = path or vendor_lib_path()
+        if not os.path.exists(self.path):
+            raise FileNotFoundError(f"{self.path} is missing: build it with `python -m cuda_hgemm_amd.build`")
+        self.dll = C.CDLL(self.path)
+        self.dll.hgemm_hipblaslt.argtypes, self.dll.hgemm_hipblaslt.restype = _HGEMM_ARGS, None
+
+    def fn(self):
+        return C.cast(self.dll.hgemm_hipblaslt, HGEMM_FN)
+
+    def call(self, A, B, C_out, M: int, N: int, K: int) -> None:
+        self.dll.hgemm_hipblaslt(_tensor_ptr(A, M, K, "A"), _tensor_ptr(B, N, K, "B"), _tensor_ptr(C_out, M, N, "C"),
+                                 M, N, K)
+
+
+_library: Optional[HgemmLibrary] = None
+_vendor: Optional[VendorLibrary] = None
+
+
+def library() -> HgemmLibrary:
+    global _library
+    if _library is None:
+        _library = HgemmLibrary()
+    return _library
+
+
+def vendor_library() -> VendorLibrary:
+    global _vendor
+    if _vendor is None:
+        _vendor = VendorLibrary()
+    return _vendor
+
+
+def hgemm(A, B, variant: str = "hgemm_auto", out=None):
+    """``C = A @ B.T`` for fp16 GPU tensors ``A (M, K)`` and ``B (N, K)`` through variant ``variant``."""
+    import torch
+    M, K = A.shape
+    N = B.shape[0]
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=A.device)
+    library().call(variant, A, B, out, M, N, K)
+    return out

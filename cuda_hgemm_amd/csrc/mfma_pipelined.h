@@ -20,9 +20,11 @@
 
 namespace hgemm {
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int GROUP_N_ = 8>
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int GROUP_N_ = 8, int DBG_ = 0>
 struct PipeConfig : TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true, GROUP_N_> {
     using Base = TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true, GROUP_N_>;
+    static constexpr int DBG = DBG_;  // timing experiments only: 1 = no copies in the loop, 2 = copies from a fixed K offset,
+                                      // 3 = 1 + no barrier, 4 = 3 + no operand reads
     static_assert(STAGES_ >= 2, "the rotated pipeline needs at least two LDS buffers");
     static bool supports(size_t M, size_t N, size_t K) {
         return M % BM_ == 0 && N % BN_ == 0 && K % BK_ == 0 && K >= (size_t)BK_ * STAGES_;
@@ -43,7 +45,7 @@ __device__ __forceinline__ void dma_load16_sv(const void *sbase, uint32_t voff, 
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_pipelined_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C, int M,
-                           int N, int K, int tiles_m, int tiles_n) {
+                           int N, int K, int tiles_m, int tiles_n, long long *trace) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, KSTEPS = Cfg::KSTEPS, CPR = Cfg::CPR;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES;
@@ -52,6 +54,8 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     static_assert(NFRAG <= NMMA, "one operand read is issued per MFMA slot");
     static_assert(KSTEPS % 2 == 0, "operand double buffer assumes an even number of steps");
     (void)M;
+    long long t_begin = 0, t_loop = 0, t_epi = 0, c_loop = 0, c_epi = 0;
+    if (Cfg::DBG == 7) t_begin = wall_clock64();
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
@@ -122,90 +126,113 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(src[TM + j], src[i], acc[i][j], 0, 0, 0);
     };
 
-    // ---- prologue: fill the whole ring, wait for chunk 0, read its first operands
+    // ---- pipeline.  Chunk c lives in ring buffer c % STAGES.
+    // SPREAD (three or more buffers): the copy of chunk kt+STAGES-1 goes into the buffer
+    // that the barrier of iteration kt-1 released and is issued one instruction at a time
+    // across all MFMA slots of iteration kt, so the texture path sees an even stream.
+    // Otherwise (two buffers): the buffer is only released by this iteration's barrier,
+    // so the copy of chunk kt+STAGES is issued across the slots of the last step.
+    constexpr bool SPREAD = STAGES >= 3;
+    constexpr int AHEAD = SPREAD ? STAGES - 1 : STAGES;      // chunk kt+AHEAD is copied in iteration kt
+    constexpr int SLOTS = SPREAD ? KSTEPS * NMMA : NMMA;     // MFMA slots the copy is spread over
+    constexpr int FIRST_SLOT = SPREAD ? 0 : (KSTEPS - 1) * NMMA;
+    // copy instructions of the current iteration already issued when its barrier is reached
+    constexpr int D_BEFORE = SPREAD ? ((KSTEPS - 1) * NMMA * L + SLOTS - 1) / SLOTS : 0;
+    // copies allowed to be still in flight at the barrier while chunk kt+1 must have landed
+    constexpr int STEADY_VMCNT = SPREAD ? (STAGES - 3) * L + D_BEFORE : (STAGES - 2) * L;
+    static_assert(STEADY_VMCNT <= 63, "vmcnt is a 6-bit counter");
+
 #pragma unroll
-    for (int s = 0; s < STAGES; ++s)
+    for (int s = 0; s < AHEAD; ++s)
 #pragma unroll
         for (int idx = 0; idx < L; ++idx) dma_one(idx, s * BK * 2, s);
-    wait_vmcnt<(STAGES - 1) * L>();
+    wait_vmcnt<(AHEAD - 1) * L>();
     __syncthreads();
 #pragma unroll
     for (int idx = 0; idx < NFRAG; ++idx) read_one(idx, 0, 0, frag[0]);
 
-    // One iteration = one K chunk.  ISSUE: a chunk remains to be copied into the buffer this
-    // iteration releases.  NEXT: another chunk follows (its operands are prefetched).
-    // STEADY: the full complement of later chunks is in flight at the barrier.
-    auto iteration = [&](int kt, int cur, auto issue_tag, auto next_tag, auto steady_tag) {
+    // One iteration = one K chunk.  ISSUE: chunk kt+AHEAD exists and is copied now.
+    // NEXT: chunk kt+1 exists (the barrier is needed and its operands are prefetched).
+    auto iteration = [&](int kt, int cur, int fill, auto issue_tag, auto next_tag) {
         constexpr bool ISSUE = decltype(issue_tag)::value, NEXT = decltype(next_tag)::value;
-        constexpr bool STEADY = decltype(steady_tag)::value;
         const int nxt = (cur + 1 == STAGES) ? 0 : cur + 1;
+        const int kbyte = (Cfg::DBG == 2 ? (kt & 1) : (kt + AHEAD)) * BK * 2;
 #pragma unroll
         for (int kk = 0; kk < KSTEPS; ++kk) {
             const int fb = (kk & 1), nb = fb ^ 1;  // KSTEPS is even: step 0 always uses frag[0]
-            if (kk + 1 < KSTEPS) {
+            const bool last = (kk + 1 == KSTEPS);
+            if (last && NEXT) {
+                if (ISSUE)
+                    wait_vmcnt<STEADY_VMCNT>();
+                else
+                    wait_vmcnt<0>();
+                if (Cfg::DBG < 3) __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
-                for (int idx = 0; idx < NMMA; ++idx) {
-                    mma_one(idx, frag[fb]);
-                    if (idx < NFRAG) read_one(idx, cur, kk + 1, frag[nb]);
-                    __builtin_amdgcn_sched_barrier(0);
+            for (int idx = 0; idx < NMMA; ++idx) {
+                mma_one(idx, frag[fb]);
+                if (idx < NFRAG && Cfg::DBG < 4) {
+                    if (!last)
+                        read_one(idx, cur, kk + 1, frag[nb]);
+                    else if (NEXT)
+                        read_one(idx, nxt, 0, frag[nb]);
                 }
-            } else {
-                if (NEXT) {
-                    if (STEADY)
-                        wait_vmcnt<(STAGES - 2) * L>();
-                    else
-                        wait_vmcnt<0>();
-                    __syncthreads();
+                if (ISSUE && (Cfg::DBG == 0 || Cfg::DBG == 2 || Cfg::DBG == 7)) {
+                    const int slot = kk * NMMA + idx - FIRST_SLOT;  // slot of this MFMA in the copy window
+#pragma unroll
+                    for (int d = 0; d < L; ++d)
+                        if (slot >= 0 && d * SLOTS / L == slot) dma_one(d, kbyte, fill);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                constexpr int DMA_PER_SLOT = (L + NMMA - 1) / NMMA;
-#pragma unroll
-                for (int idx = 0; idx < NMMA; ++idx) {
-                    mma_one(idx, frag[fb]);
-                    if (NEXT && idx < NFRAG) read_one(idx, nxt, 0, frag[nb]);
-                    if (ISSUE) {
-#pragma unroll
-                        for (int d = 0; d < DMA_PER_SLOT; ++d)
-                            if (idx * DMA_PER_SLOT + d < L)
-                                dma_one(idx * DMA_PER_SLOT + d, (kt + STAGES) * BK * 2, cur);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                }
             }
         }
     };
+    if (Cfg::DBG == 7) {
+        t_loop = wall_clock64();
+        c_loop = clock64();
+    }
     using T = std::true_type;
     using F = std::false_type;
 
-    int kt = 0, cur = 0;
-    for (; kt < num_k - STAGES; ++kt) {  // chunks kt+STAGES exist
-        iteration(kt, cur, T{}, T{}, T{});
+    int kt = 0, cur = 0, fill = SPREAD ? STAGES - 1 : 0;
+    auto advance = [&] {
         cur = (cur + 1 == STAGES) ? 0 : cur + 1;
+        fill = (fill + 1 == STAGES) ? 0 : fill + 1;
+    };
+    for (; kt < num_k - AHEAD; ++kt) {  // chunk kt+AHEAD exists
+        iteration(kt, cur, fill, T{}, T{});
+        advance();
     }
     for (; kt < num_k - 1; ++kt) {  // drain: nothing left to copy
-        iteration(kt, cur, F{}, T{}, F{});
-        cur = (cur + 1 == STAGES) ? 0 : cur + 1;
+        iteration(kt, cur, fill, F{}, T{});
+        advance();
     }
-    iteration(kt, cur, F{}, F{}, F{});
+    iteration(kt, cur, fill, F{}, F{});
 
-    // ---- epilogue: accumulators -> fp16 -> C
-    half_t *Cw = C + (size_t)(tile_m * BM + wm * Cfg::WM + (lane & 31)) * N + tile_n * BN + wn * Cfg::WN +
-                 ((lane >> 5) << 2);
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                half4 v;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) v[r] = (half_t)acc[i][j][g * 4 + r];
-                *reinterpret_cast<half4 *>(Cw + (size_t)i * 32 * N + j * 32 + g * 8) = v;
-            }
+    // ---- epilogue: accumulators -> fp16 -> C (through LDS, whole lines per store)
+    if (Cfg::DBG == 7) {
+        t_epi = wall_clock64();
+        c_epi = clock64();
+    }
+    __syncthreads();
+    store_tile_via_lds<Cfg>(acc, lds, C, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN, wave, lane);
+    if (Cfg::DBG == 7 && trace && tid == 0) {
+        __builtin_amdgcn_s_waitcnt(0);
+        long long *t = trace + (size_t)blockIdx.x * 8;
+        t[0] = t_begin;
+        t[1] = t_loop;
+        t[2] = t_epi;
+        t[3] = wall_clock64();
+        t[4] = __builtin_amdgcn_s_getreg((31 << 11) | 4);   // HW_ID: wave / simd / cu / sh / se
+        t[5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID
+        t[6] = c_epi - c_loop;
+    }
 }
 
 template <class Cfg>
-void launch_pipelined(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, const char *name) {
+void launch_pipelined(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, const char *name,
+                      long long *trace = nullptr) {
     check_operands(A, B, C, M, N, K);
     HGEMM_CHECK_MSG(Cfg::supports(M, N, K),
                     "%s needs M %% %d == 0, N %% %d == 0, K %% %d == 0, K >= %d (got M=%zu N=%zu K=%zu)", name,
@@ -219,7 +246,7 @@ void launch_pipelined(const void *A, const void *B, void *C, size_t M, size_t N,
     const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
     hgemm_pipelined_kernel<Cfg><<<dim3(tiles_m * tiles_n), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
-        (int)M, (int)N, (int)K, tiles_m, tiles_n);
+        (int)M, (int)N, (int)K, tiles_m, tiles_n, trace);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 

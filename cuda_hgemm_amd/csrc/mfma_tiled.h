@@ -55,7 +55,10 @@ struct TileConfig {
     static constexpr int ROW_BYTES = BK * 2 + (LAYOUT == LDS_PADDED ? 16 : 0);
     static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-    static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+    static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
+    // the C tile is staged through LDS on its way out: one 32-row strip per wave
+    static constexpr int C_STRIP_BYTES = 32 * (WN * 2 + 16);
+    static constexpr int LDS_BYTES = RING_BYTES > WAVES * C_STRIP_BYTES ? RING_BYTES : WAVES * C_STRIP_BYTES;
     // register-staged copy: each thread moves this many 16-byte chunks per tile
     static constexpr int A_ITERS = BM * CPR / THREADS, B_ITERS = BN * CPR / THREADS;
     // direct-to-LDS copy: one wave instruction fills 1024 contiguous LDS bytes
@@ -128,6 +131,49 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
     const int width = (tiles_n - n_first) < Cfg::GROUP_N ? (tiles_n - n_first) : Cfg::GROUP_N;
     tile_m = within / width;
     tile_n = n_first + within % width;
+}
+
+// Epilogue shared by the tiled kernels: accumulators -> fp16 -> C, staged through LDS.
+// A lane of the (operand-swapped) accumulator holds four consecutive n of one row; stored
+// straight to global memory that is 16 useful bytes per 32 rows per instruction, i.e. a
+// flood of partial-line write requests.  Instead each wave parks 32 rows of its tile in a
+// private LDS strip (row stride WN*2 + 16 bytes) and reads them back row-contiguous, so
+// every global store instruction writes whole 128-byte lines, 16 bytes per lane.
+// The caller must have passed a workgroup barrier after the last operand read, because
+// the strips reuse the operand buffers.
+template <class Cfg>
+__device__ __forceinline__ void store_tile_via_lds(const floatx16 (&acc)[Cfg::TM][Cfg::TN], unsigned char *lds,
+                                                   half_t *__restrict__ C, int N, int row0, int col0, int wave,
+                                                   int lane) {
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, WN = Cfg::WN;
+    constexpr int STRIP_ROW_BYTES = WN * 2 + 16;
+    constexpr int STRIP_BYTES = 32 * STRIP_ROW_BYTES;
+    constexpr int LANES_PER_ROW = WN / 8;            // 16-byte pieces per row
+    constexpr int ROWS_PER_READ = 64 / LANES_PER_ROW;
+    constexpr int READS = 32 / ROWS_PER_READ;
+    static_assert(STRIP_BYTES == Cfg::C_STRIP_BYTES, "strip size");
+    unsigned char *strip = lds + wave * STRIP_BYTES;
+    unsigned char *wr = strip + (lane & 31) * STRIP_ROW_BYTES + ((lane >> 5) << 3);
+    const int rd_row = lane / LANES_PER_ROW, rd_col = lane % LANES_PER_ROW;
+    const unsigned char *rd = strip + rd_row * STRIP_ROW_BYTES + rd_col * 16;
+    half_t *cp = C + (size_t)(row0 + rd_row) * N + col0 + rd_col * 8;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                half4 v;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = (half_t)acc[i][j][g * 4 + r];
+                *reinterpret_cast<half4 *>(wr + (j * 32 + g * 8) * 2) = v;
+            }
+#pragma unroll
+        for (int it = 0; it < READS; ++it) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(rd + it * ROWS_PER_READ * STRIP_ROW_BYTES);
+            *reinterpret_cast<u32x4 *>(cp + (size_t)(i * 32 + it * ROWS_PER_READ) * N) = v;
+        }
+    }
 }
 
 template <class Cfg>
@@ -322,19 +368,8 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     }
 
     // ---------------- epilogue: accumulators -> fp16 -> C ----------------
-    half_t *Cw = C + (size_t)(tile_m * BM + wm * Cfg::WM + (lane & 31)) * N + tile_n * BN + wn * Cfg::WN +
-                 ((lane >> 5) << 2);
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                half4 v;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) v[r] = (half_t)acc[i][j][g * 4 + r];
-                *reinterpret_cast<half4 *>(Cw + (size_t)i * 32 * N + j * 32 + g * 8) = v;
-            }
+    __syncthreads();
+    store_tile_via_lds<Cfg>(acc, lds, C, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN, wave, lane);
 }
 
 // Host launcher shared by every tiled entry point.  Sets the dynamic-LDS limit once per

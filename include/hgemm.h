@@ -89,6 +89,11 @@ HGEMM_FUNC(hgemm_skinny);
  * This is the entry point the benchmark measures. */
 HGEMM_FUNC(hgemm_auto);
 
+/* Kernel hgemm_auto would pick for a shape (an id for hgemm_kernel_name) and, through
+ * `splits` if not NULL, the number of K slices; no launch happens. */
+int hgemm_auto_plan(size_t M, size_t N, size_t K, int *splits);
+const char *hgemm_kernel_name(int kernel);
+
 /* ---- registry, so a driver can enumerate variants the way the reference's main lists
  * them (reference src/main.cu:100-123) without an edit per variant. ---- */
 int hgemm_variant_count(void);

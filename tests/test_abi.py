@@ -1,0 +1,150 @@
+"""The C-ABI boundary without a GPU: the library loads, exports every symbol the headers
+declare, its registry and shape predicates answer, and contract violations end the
+process with a message (the convention of the reference's HGEMM_CHECK macros,
+src/common/common.h:23-29) before any GPU call."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+INCLUDE = os.path.join(ROOT, "include")
+
+
+def _declared_symbols(header):
+    text = open(os.path.join(INCLUDE, header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = set(re.findall(r"^HGEMM_FUNC\((\w+)\);", text, flags=re.M))
+    names |= set(re.findall(r"^(?:const\s+)?\w[\w\s\*]*?\b(hgemm_\w+)\s*\(", text, flags=re.M))
+    names.discard("hgemm_fn")
+    return names
+
+
+def test_library_exports_every_declared_symbol(hgemm_lib):
+    declared = _declared_symbols("hgemm.h")
+    assert len(declared) >= 25, declared
+    for name in sorted(declared):
+        assert hasattr(hgemm_lib.dll, name), f"libhgemm.so does not export {name}"
+    from cuda_hgemm_amd.binding import HELPER_SYMBOLS, KERNEL_SYMBOLS
+    assert declared == set(KERNEL_SYMBOLS) | set(HELPER_SYMBOLS)
+
+
+def test_vendor_library_exports_its_symbol(vendor_lib):
+    assert _declared_symbols("hgemm_hipblaslt.h") == {"hgemm_hipblaslt"}
+    assert hasattr(vendor_lib.dll, "hgemm_hipblaslt")
+
+
+def test_measured_library_has_no_blas_dependency(hgemm_lib):
+    out = subprocess.run(["ldd", hgemm_lib.path], capture_output=True, text=True).stdout
+    assert "blas" not in out.lower(), out
+    assert "libamdhip64" in out
+
+
+def test_registry(hgemm_lib):
+    variants = hgemm_lib.variants()
+    names = [v["name"] for v in variants]
+    assert names[0] == "Simt-Naive" and "Mfma-Async-Stage4" in names and names[-1] == "Auto"
+    assert len(set(names)) == len(names)
+    for v in variants:
+        assert hgemm_lib.find(v["name"]) == v["index"] == hgemm_lib.find(v["symbol"])
+        assert hasattr(hgemm_lib.dll, v["symbol"])
+    # the naive / base kernels are left out of the default run, as in the reference's main
+    assert [v["name"] for v in variants if not v["default_run"]] == ["Simt-Naive", "Mfma-Naive", "Mfma-Base"]
+    with pytest.raises(KeyError):
+        hgemm_lib.find("no-such-variant")
+
+
+def test_shape_predicates(hgemm_lib):
+    s = hgemm_lib.supports
+    assert s("hgemm_simt_naive", 1, 1, 1) and s("hgemm_auto", 100, 100, 100)
+    assert s("hgemm_mfma_naive", 32, 64, 16) and not s("hgemm_mfma_naive", 32, 64, 8)
+    # 256 x 128 x 32 tiles, as the reference's kernels (src/mma/mma_async_stage4.cu:13-14)
+    for name in ("hgemm_mfma_base", "hgemm_mfma_padding", "hgemm_mfma_swizzle", "hgemm_mfma_async",
+                 "hgemm_mfma_async_pg2s", "hgemm_mfma_async_pg2s_ps2r", "hgemm_mfma_async_stage3",
+                 "hgemm_mfma_async_stage4"):
+        assert s(name, 256, 128, 256) and s(name, 512, 2048, 1024)
+        assert not s(name, 128, 128, 256) and not s(name, 256, 64, 256) and not s(name, 256, 128, 48)
+    assert not s("hgemm_mfma_async_stage4", 256, 128, 64)      # K must cover the 3-chunk prologue
+    assert s("hgemm_mfma_async_stage4", 256, 128, 96)
+    assert s("hgemm_skinny", 1, 4096, 4096) and s("hgemm_skinny", 128, 28672, 4096)
+    assert not s("hgemm_skinny", 129, 4096, 4096) and not s("hgemm_skinny", 8, 100, 4096)
+    assert not s("hgemm_auto", 0, 8, 8) and not s("hgemm_auto", 1 << 20, 8, 1 << 20)
+
+
+def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
+    plan = hgemm_lib.auto_plan
+    for n in (256, 512, 1024, 2048, 4096, 8192, 16384):
+        p = plan(n, n, n)
+        assert p["kernel"] != "scalar fallback" and p["splits"] >= 1, (n, p)
+    assert plan(8192, 8192, 8192)["kernel"].startswith("pipelined 256x256")
+    for shape in ((4096, 14336, 4096), (4096, 4096, 14336)):
+        assert plan(*shape)["kernel"].startswith("pipelined"), shape
+    for m in (1, 8, 16, 64, 128):
+        for n in (4096, 28672):
+            p = plan(m, n, 4096)
+            assert p["kernel"].startswith("split-K"), (m, n, p)
+            assert 4096 % (p["splits"] * 64) == 0
+    assert plan(100, 100, 100)["kernel"] == "scalar fallback"
+
+
+def test_metrics(hgemm_lib):
+    assert abs(hgemm_lib.tflops(8192, 8192, 8192, 1.0) - 1099.511627776) < 1e-9
+    assert hgemm_lib.bytes(8192, 8192, 8192) == 2.0 * 3 * 8192 * 8192
+    assert hgemm_lib.bytes(1, 4096, 4096) == 2.0 * (4096 + 4096 * 4096 + 4096)
+    assert "gfx950" in hgemm_lib.version()
+
+
+_VIOLATION = r"""
+import ctypes, sys
+sys.path.insert(0, {root!r})
+import cuda_hgemm_amd
+L = cuda_hgemm_amd.library()
+buf = ctypes.create_string_buffer(64)
+p = ctypes.addressof(buf)
+{call}
+print("returned")
+"""
+
+
+@pytest.mark.parametrize("call,needle", [
+    ("L.dll.hgemm_auto(None, p, p, 8, 8, 8)", "Check failed: A != nullptr"),
+    ("L.dll.hgemm_auto(p, p, p, 0, 8, 8)", "Check failed: (M) > (0u)"),
+    ("L.dll.hgemm_mfma_async_stage4(p, p, p, 100, 128, 256)", "needs M % 256 == 0"),
+    ("L.dll.hgemm_mfma_naive(p, p, p, 32, 32, 8)", "K % 16 == 0"),
+    ("L.dll.hgemm_skinny(p, p, p, 200, 4096, 4096)", "M <= 128"),
+    ("L.dll.hgemm_variant_name(99)", "out of range"),
+])
+def test_contract_violation_ends_the_process_with_a_message(call, needle):
+    """No GPU call is reached: the checks run first, so this is safe on a CPU-only box."""
+    code = _VIOLATION.format(root=ROOT, call=call)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 1, (r.returncode, r.stdout, r.stderr)
+    assert "returned" not in r.stdout
+    assert needle in r.stderr and "[HGEMM " in r.stderr, r.stderr
+
+
+def test_binding_rejects_bad_tensors(hgemm_lib):
+    import torch
+    a = torch.zeros((8, 8), dtype=torch.float16)
+    with pytest.raises(ValueError, match="must live on the GPU"):
+        hgemm_lib.call("hgemm_auto", a, a, a, 8, 8, 8)
+    with pytest.raises(TypeError, match="float16"):
+        hgemm_lib.call("hgemm_auto", a.float(), a, a, 8, 8, 8)
+
+
+def test_driver_flag_parser():
+    from cuda_hgemm_amd import driver_path
+    exe = driver_path()
+    assert os.path.exists(exe), "build the driver with `python -m cuda_hgemm_amd.build`"
+    r = subprocess.run([exe, "-help"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0
+    for flag in ("-M ", "-N ", "-K ", "-warmup_iterations", "-profiling_iterations", "-sleep_duration", "-enable_check",
+                 "-cpu_procs", "-gpu_rank", "-seed", "-dist_a", "-dist_b"):
+        assert flag in r.stderr, flag
+    r = subprocess.run([exe, "-no_such_flag=1"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 1 and "unknown flag -no_such_flag" in r.stderr
+    r = subprocess.run([exe, "-M=abc"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 1 and "is not a count" in r.stderr
