@@ -44,6 +44,17 @@ HELPER_SYMBOLS = [
 ]
 
 
+def _share_hip_runtime_with_torch() -> None:
+    """PyTorch wheels carry their own libamdhip64 (same soname as the system one).  Two HIP
+    runtimes in one process do not share devices or memory, so torch must be loaded first:
+    the dynamic linker then resolves this library's libamdhip64 dependency to the copy that
+    is already mapped, and tensors and kernels live in one runtime."""
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass  # a caller without torch brings its own device pointers and the system runtime
+
+
 def _tensor_ptr(t, rows: int, cols: int, what: str) -> int:
     import torch
     if not isinstance(t, torch.Tensor):
@@ -68,6 +79,7 @@ class HgemmLibrary:
             raise FileNotFoundError(
                 f"{self.path} is missing: build it with `python -m cuda_hgemm_amd.build` (needs hipcc); "
                 "there is no non-HIP fallback")
+        _share_hip_runtime_with_torch()
         self.dll = C.CDLL(self.path)
         d = self.dll
         for name in KERNEL_SYMBOLS:
@@ -169,6 +181,7 @@ class VendorLibrary:
         self.path = path or vendor_lib_path()
         if not os.path.exists(self.path):
             raise FileNotFoundError(f"{self.path} is missing: build it with `python -m cuda_hgemm_amd.build`")
+        _share_hip_runtime_with_torch()
         self.dll = C.CDLL(self.path)
         self.dll.hgemm_hipblaslt.argtypes, self.dll.hgemm_hipblaslt.restype = _HGEMM_ARGS, None
 
