@@ -15,47 +15,164 @@
 #pragma once
 
 #include <type_traits>
+#include <utility>
 
 #include "mfma_tiled.h"
 
 namespace hgemm {
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int GROUP_N_ = 8, int DBG_ = 0>
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int MI_ = 16, int GROUP_N_ = 8,
+          int DBG_ = 0>
 struct PipeConfig : TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true, GROUP_N_> {
     using Base = TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true, GROUP_N_>;
-    static constexpr int DBG = DBG_;  // timing experiments only: 1 = no copies in the loop, 2 = copies from a fixed K offset,
-                                      // 3 = 1 + no barrier, 4 = 3 + no operand reads
+    // MFMA shape: 32 -> v_mfma_f32_32x32x16_f16, 16 -> v_mfma_f32_16x16x32_f16.  Both move
+    // the same bytes from LDS per flop (that depends on the wave tile only); the 16x16x32
+    // form reads and writes half as many accumulator registers per flop and sustains a
+    // higher clock under the board's power limit.
+    static constexpr int MI = MI_;
+    static constexpr int PTM = Base::WM / MI, PTN = Base::WN / MI;  // MFMA tiles per wave
+    static constexpr int PKSTEP = MI == 32 ? 16 : 32;               // k covered by one MFMA
+    static constexpr int PKSTEPS = BK_ / PKSTEP;
+    static constexpr int CPS = PKSTEP / 8;                          // 16-byte chunks per row per step
+    // timing experiments only: 1 = no copies in the loop, 2 = copies from a fixed K offset,
+    // 4 = no operand reads in the loop.  (Per-workgroup timestamps are written whenever the
+    // launcher is given a trace buffer.)
+    static constexpr int DBG = DBG_;
+    static_assert(MI == 16 || MI == 32, "MFMA tile is 16x16x32 or 32x32x16");
     static_assert(STAGES_ >= 2, "the rotated pipeline needs at least two LDS buffers");
+    static_assert(Base::WM % MI == 0 && Base::WN % MI == 0, "wave tile must be a multiple of the MFMA tile");
+    static_assert(PKSTEPS % 2 == 0, "the operand double buffer needs an even number of MFMA steps per chunk");
     static bool supports(size_t M, size_t N, size_t K) {
         return M % BM_ == 0 && N % BN_ == 0 && K % BK_ == 0 && K >= (size_t)BK_ * STAGES_;
     }
 };
 
-// Direct-to-LDS copy, scalar base + 32-bit per-lane byte offset.
-__device__ __forceinline__ void dma_load16_sv(const void *sbase, uint32_t voff, uint32_t lds_addr) {
+// Compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>).  The
+// pipeline body is laid out slot by slot with every index a constant; this does not lean
+// on the loop unroller, whose failure would turn the accumulators into scratch memory.
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(static_cast<F &&>(f), std::make_integer_sequence<int, N>{});
+}
+
+// LDS operand read and its wait, written as assembly: the optimiser moves ordinary LDS loads
+// freely (it batched them at the top of the loop, which both breaks the interleave with
+// the MFMAs and blows the register budget), so the reads are pinned here and the kernel
+// does its own lgkmcnt accounting.  lds_wait_all ties the fragment registers through the
+// wait so no MFMA that consumes them can be scheduled above it.
+template <int OFFSET>
+__device__ __forceinline__ half8 lds_read16(uint32_t addr) {
+    half8 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFFSET));
+    return v;
+}
+__device__ __forceinline__ void lds_wait_all(half8 &a, half8 &b, half8 &c, half8 &d) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+__device__ __forceinline__ void lds_wait_all(half8 &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a)); }
+
+// The MFMA itself is issued from assembly too, with the accumulator pinned to AGPRs: that
+// fixes the order of MFMAs, operand reads and copies exactly as written (volatile
+// statements are never reordered against each other) and keeps the register allocator from
+// shuttling accumulators between the two register files.  The kernel guarantees what the
+// compiler no longer checks: an accumulator is reused only a full step (>= 16 MFMAs) later,
+// and operands are covered by lds_wait_all.
+template <int MI>
+struct MfmaOp;
+template <>
+struct MfmaOp<32> {
+    typedef floatx16 Acc;
+    static constexpr int REGS = 16;
+    static __device__ __forceinline__ void run(half8 a, half8 b, Acc &c) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+};
+template <>
+struct MfmaOp<16> {
+    typedef floatx4 Acc;
+    static constexpr int REGS = 4;
+    static __device__ __forceinline__ void run(half8 a, half8 b, Acc &c) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+};
+
+// Ordered no-op that "modifies" an accumulator: later reads of it stay behind this point.
+template <class Acc>
+__device__ __forceinline__ void pin_accumulator(Acc &c) {
+    asm volatile("" : "+a"(c));
+}
+
+// Direct-to-LDS copy: global address = scalar base + 32-bit per-lane byte offset, LDS
+// destination (wave-uniform, goes through M0) = lds_base + LDS_IMM.
+template <int LDS_IMM>
+__device__ __forceinline__ void dma_load16_sv(const void *sbase, uint32_t voff, uint32_t lds_base) {
     asm volatile(
-        "s_mov_b32 m0, %0\n\t"
+        "s_add_u32 m0, %0, %3\n\t"
         "s_nop 0\n\t"
         "global_load_lds_dwordx4 %1, %2"
         :
-        : "s"(lds_addr), "v"(voff), "s"(sbase)
-        : "memory");
+        : "s"(lds_base), "v"(voff), "s"(sbase), "i"(LDS_IMM)
+        : "memory", "scc");
+}
+
+// Accumulators -> fp16 -> C through LDS for either MFMA shape (operands swapped, so a lane
+// holds groups of four consecutive n of one row m = lane % MI): each wave parks MI rows of
+// its tile in a private strip and reads them back row-contiguous, 16 bytes per lane, so a
+// global store instruction writes whole 128-byte lines.
+template <class Cfg, class Acc>
+__device__ __forceinline__ void store_wave_tile(const Acc (&acc)[Cfg::PTM][Cfg::PTN], unsigned char *lds,
+                                                half_t *__restrict__ C, int N, int row0, int col0, int wave,
+                                                int lane) {
+    constexpr int MI = Cfg::MI, TM = Cfg::PTM, TN = Cfg::PTN, WN = Cfg::WN;
+    constexpr int GROUPS = MI == 32 ? 4 : 1;          // register groups of four n per accumulator
+    constexpr int STRIP_ROW_BYTES = WN * 2 + 16;
+    constexpr int STRIP_BYTES = 32 * STRIP_ROW_BYTES;  // sized for the 32-row case
+    constexpr int LANES_PER_ROW = WN / 8;
+    constexpr int ROWS_PER_READ = 64 / LANES_PER_ROW;
+    constexpr int READS = MI / ROWS_PER_READ;
+    static_assert(STRIP_BYTES == Cfg::C_STRIP_BYTES, "strip size");
+    unsigned char *strip = lds + wave * STRIP_BYTES;
+    unsigned char *wr = strip + (lane % MI) * STRIP_ROW_BYTES + ((lane / MI) << 3);
+    const int rd_row = lane / LANES_PER_ROW, rd_col = lane % LANES_PER_ROW;
+    const unsigned char *rd = strip + rd_row * STRIP_ROW_BYTES + rd_col * 16;
+    half_t *cp = C + (size_t)(row0 + rd_row) * N + col0 + rd_col * 8;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int g = 0; g < GROUPS; ++g) {
+                half4 v;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = (half_t)acc[i][j][g * 4 + r];
+                *reinterpret_cast<half4 *>(wr + (j * MI + g * 8) * 2) = v;
+            }
+#pragma unroll
+        for (int it = 0; it < READS; ++it) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(rd + it * ROWS_PER_READ * STRIP_ROW_BYTES);
+            *reinterpret_cast<u32x4 *>(cp + (size_t)(i * MI + it * ROWS_PER_READ) * N) = v;
+        }
+    }
 }
 
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_pipelined_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C, int M,
                            int N, int K, int tiles_m, int tiles_n, long long *trace) {
-    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
-    constexpr int TM = Cfg::TM, TN = Cfg::TN, KSTEPS = Cfg::KSTEPS, CPR = Cfg::CPR;
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
+    constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS, CPR = Cfg::CPR, CPS = Cfg::CPS;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES;
     constexpr int A_DMA = Cfg::A_DMA, B_DMA = Cfg::B_DMA, L = A_DMA + B_DMA;
     constexpr int NFRAG = TM + TN, NMMA = TM * TN;
-    static_assert(NFRAG <= NMMA, "one operand read is issued per MFMA slot");
-    static_assert(KSTEPS % 2 == 0, "operand double buffer assumes an even number of steps");
+    typedef typename MfmaOp<MI>::Acc Acc;
+    static_assert(NFRAG <= NMMA, "at most one operand read is issued per MFMA slot");
     (void)M;
     long long t_begin = 0, t_loop = 0, t_epi = 0, c_loop = 0, c_epi = 0;
-    if (Cfg::DBG == 7) t_begin = wall_clock64();
+    if (trace) t_begin = wall_clock64();
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
@@ -78,52 +195,97 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         const int row = wave * Cfg::ROWS_PER_DMA + lane / CPR;
         const int ch = (lane % CPR) ^ swizzle_of_row<Cfg>(row);
 #pragma unroll
-        for (int it = 0; it < A_DMA; ++it) voff[it] = ((uint32_t)(row + it * DMA_ROW_STEP) * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
+        for (int it = 0; it < A_DMA; ++it)
+            voff[it] = ((uint32_t)(row + it * DMA_ROW_STEP) * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
 #pragma unroll
         for (int it = 0; it < B_DMA; ++it)
             voff[A_DMA + it] = ((uint32_t)(row + it * DMA_ROW_STEP) * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
     }
     const uint32_t cp_lds = lds_base + wave * 1024;
     // copy instruction `idx` (0..L-1) of chunk at byte offset kbyte into ring buffer `stage`
-    auto dma_one = [&](int idx, int kbyte, int stage) {
-        const uint32_t dst = cp_lds + stage * Cfg::STAGE_BYTES;
-        if (idx < A_DMA)
-            dma_load16_sv(a_base + kbyte, voff[idx], dst + idx * Cfg::WAVES * 1024);
+    // `a_src` / `b_src` already point at the chunk; `dst` is cp_lds + stage * STAGE_BYTES
+    auto dma_one = [&](auto idx_c, const unsigned char *a_src, const unsigned char *b_src, uint32_t dst) {
+        constexpr int idx = decltype(idx_c)::value;
+        if constexpr (idx < A_DMA)
+            dma_load16_sv<idx * Cfg::WAVES * 1024>(a_src, voff[idx], dst);
         else
-            dma_load16_sv(b_base + kbyte, voff[idx], dst + Cfg::A_BYTES + (idx - A_DMA) * Cfg::WAVES * 1024);
+            dma_load16_sv<Cfg::A_BYTES + (idx - A_DMA) * Cfg::WAVES * 1024>(b_src, voff[idx], dst);
     };
 
-    // ---- operand fragment set-up
-    const int frag_row = lane & 31;
-    const int frag_x = (lane >> 5) ^ swizzle_of_row<Cfg>(frag_row);
+    // ---- operand fragment set-up: lane l supplies 8 consecutive k (chunk l / MI of the
+    // step) of row l % MI, for both operands.
+    const int frag_row = lane % MI;
+    const int frag_x = (lane / MI) ^ swizzle_of_row<Cfg>(frag_row);
     const uint32_t a_frag_off = (wm * Cfg::WM + frag_row) * ROW_BYTES;
     const uint32_t b_frag_off = Cfg::A_BYTES + (wn * Cfg::WN + frag_row) * ROW_BYTES;
-    uint32_t chunk_off[KSTEPS];
+    // Fragment idx sits idx * MI rows further down.  That never changes bits 0-2 of the
+    // row's bank-line index, and changes bit 3 (which the swizzle folds into bit 0) only
+    // when MI rows are 8 lines: then odd fragments use the chunk index XOR 1.
+    constexpr int ODD_FLIP = ((MI * BK * 2 / 128) % 16 == 8) ? 16 : 0;
+    uint32_t chunk_off[KSTEPS][ODD_FLIP ? 2 : 1];
 #pragma unroll
-    for (int kk = 0; kk < KSTEPS; ++kk) chunk_off[kk] = (uint32_t)((kk * 2) ^ frag_x) << 4;
+    for (int kk = 0; kk < KSTEPS; ++kk) {
+        chunk_off[kk][0] = (uint32_t)((kk * CPS) ^ frag_x) << 4;
+        if (ODD_FLIP) chunk_off[kk][ODD_FLIP ? 1 : 0] = chunk_off[kk][0] ^ ODD_FLIP;
+    }
 
-    half8 frag[2][NFRAG];  // [buffer][A fragments 0..TM-1, then B fragments]
-    // fragment read number `idx` (0..NFRAG-1) of step kk of ring buffer `stage`
-    auto read_one = [&](int idx, int stage, int kk, half8 (&dst)[NFRAG]) {
-        const unsigned char *s = lds + stage * Cfg::STAGE_BYTES + chunk_off[kk];
-        if (idx < TM)
-            dst[idx] = *reinterpret_cast<const half8 *>(s + a_frag_off + idx * 32 * ROW_BYTES);
-        else
-            dst[idx] = *reinterpret_cast<const half8 *>(s + b_frag_off + (idx - TM) * 32 * ROW_BYTES);
+    // Operand registers.  MFMAs run B-major (all A tiles against B tile 0, then B tile 1,
+    // ...): a B fragment is dead after TM MFMAs and is reloaded in place for the next step
+    // right away, so only the A fragments (needed for the whole step) and the last B
+    // fragment are double buffered.  This keeps the kernel well inside the register file
+    // next to 256 accumulator registers.
+    half8 a_frag[2][TM];
+    constexpr int NDB = 2;                 // trailing B tiles that are double buffered
+    constexpr int NSB = TN - NDB;          // leading B tiles reloaded in place
+    half8 b_frag[NSB > 0 ? NSB : 1];
+    half8 b_last[2][NDB];
+    // Byte address (32-bit LDS offset) of this lane's fragment of A tile 0 / B tile 0 for
+    // step kk, without the ring-buffer base; tile t adds the constant t * MI * ROW_BYTES.
+    uint32_t a_addr[KSTEPS][ODD_FLIP ? 2 : 1], b_addr[KSTEPS][ODD_FLIP ? 2 : 1];
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; ++kk)
+#pragma unroll
+        for (int f = 0; f < (ODD_FLIP ? 2 : 1); ++f) {
+            a_addr[kk][f] = lds_base + a_frag_off + chunk_off[kk][f];
+            b_addr[kk][f] = lds_base + b_frag_off + chunk_off[kk][f];
+        }
+    static_assert(Cfg::A_BYTES + (TN - 1) * MI * ROW_BYTES < 65536 && (TM - 1) * MI * ROW_BYTES < 65536,
+                  "fragment offsets must fit the 16-bit ds_read offset field");
+    auto read_a = [&](auto t_c, uint32_t stage_bytes, auto kk_c) -> half8 {
+        constexpr int t = decltype(t_c)::value, kk = decltype(kk_c)::value;
+        return lds_read16<t * MI * ROW_BYTES>(a_addr[kk][ODD_FLIP ? (t & 1) : 0] + stage_bytes);
+    };
+    auto read_b = [&](auto t_c, uint32_t stage_bytes, auto kk_c) -> half8 {
+        constexpr int t = decltype(t_c)::value, kk = decltype(kk_c)::value;
+        return lds_read16<t * MI * ROW_BYTES>(b_addr[kk][ODD_FLIP ? (t & 1) : 0] + stage_bytes);
+    };
+    // every outstanding operand read has landed; ties all fragments of buffer `buf`
+    auto wait_operands = [&](auto buf_c) {
+        constexpr int buf = decltype(buf_c)::value;
+        static_for<TM / 4>([&](auto g) {
+            constexpr int t = decltype(g)::value * 4;
+            lds_wait_all(a_frag[buf][t], a_frag[buf][t + 1], a_frag[buf][t + 2], a_frag[buf][t + 3]);
+        });
+        static_for<NSB>([&](auto t) { lds_wait_all(b_frag[decltype(t)::value]); });
+        static_for<NDB>([&](auto t) { lds_wait_all(b_last[buf][decltype(t)::value]); });
     };
 
-    floatx16 acc[TM][TN];
+    Acc acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+            for (int r = 0; r < MfmaOp<MI>::REGS; ++r) acc[i][j][r] = 0.0f;
 
-    auto mma_one = [&](int idx, const half8 (&src)[NFRAG]) {
-        const int i = idx / TN;
-        const int j = (i & 1) ? (TN - 1 - idx % TN) : (idx % TN);  // serpentine
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(src[TM + j], src[i], acc[i][j], 0, 0, 0);
+    // MFMA slot idx of a step: B tile idx / TM against A tile idx % TM, from buffer fb.
+    auto mma_one = [&](auto idx_c, auto fb_c) {
+        constexpr int idx = decltype(idx_c)::value, fb = decltype(fb_c)::value;
+        constexpr int j = idx / TM, i = idx % TM;
+        if constexpr (j >= NSB)
+            MfmaOp<MI>::run(b_last[fb][j - NSB], a_frag[fb][i], acc[i][j]);
+        else
+            MfmaOp<MI>::run(b_frag[j], a_frag[fb][i], acc[i][j]);
     };
 
     // ---- pipeline.  Chunk c lives in ring buffer c % STAGES.
@@ -136,20 +298,28 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     constexpr int AHEAD = SPREAD ? STAGES - 1 : STAGES;      // chunk kt+AHEAD is copied in iteration kt
     constexpr int SLOTS = SPREAD ? KSTEPS * NMMA : NMMA;     // MFMA slots the copy is spread over
     constexpr int FIRST_SLOT = SPREAD ? 0 : (KSTEPS - 1) * NMMA;
+    static_assert(TM >= 4 && TN >= 2, "the operand schedule needs at least 4 x 2 MFMA tiles per wave");
     // copy instructions of the current iteration already issued when its barrier is reached
     constexpr int D_BEFORE = SPREAD ? ((KSTEPS - 1) * NMMA * L + SLOTS - 1) / SLOTS : 0;
     // copies allowed to be still in flight at the barrier while chunk kt+1 must have landed
     constexpr int STEADY_VMCNT = SPREAD ? (STAGES - 3) * L + D_BEFORE : (STAGES - 2) * L;
     static_assert(STEADY_VMCNT <= 63, "vmcnt is a 6-bit counter");
 
-#pragma unroll
-    for (int s = 0; s < AHEAD; ++s)
-#pragma unroll
-        for (int idx = 0; idx < L; ++idx) dma_one(idx, s * BK * 2, s);
+    static_for<AHEAD>([&](auto s_c) {
+        constexpr int st = decltype(s_c)::value;
+        static_for<L>([&](auto idx_c) {
+            dma_one(idx_c, a_base + st * BK * 2, b_base + st * BK * 2, cp_lds + st * Cfg::STAGE_BYTES);
+        });
+    });
     wait_vmcnt<(AHEAD - 1) * L>();
     __syncthreads();
-#pragma unroll
-    for (int idx = 0; idx < NFRAG; ++idx) read_one(idx, 0, 0, frag[0]);
+    using K0 = std::integral_constant<int, 0>;
+    static_for<TM>([&](auto t) { a_frag[0][decltype(t)::value] = read_a(t, 0u, K0{}); });
+    static_for<NSB>([&](auto t) { b_frag[decltype(t)::value] = read_b(t, 0u, K0{}); });
+    static_for<NDB>([&](auto t) {
+        b_last[0][decltype(t)::value] = read_b(std::integral_constant<int, NSB + decltype(t)::value>{}, 0u, K0{});
+    });
+    wait_operands(std::integral_constant<int, 0>{});
 
     // One iteration = one K chunk.  ISSUE: chunk kt+AHEAD exists and is copied now.
     // NEXT: chunk kt+1 exists (the barrier is needed and its operands are prefetched).
@@ -157,38 +327,57 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         constexpr bool ISSUE = decltype(issue_tag)::value, NEXT = decltype(next_tag)::value;
         const int nxt = (cur + 1 == STAGES) ? 0 : cur + 1;
         const int kbyte = (Cfg::DBG == 2 ? (kt & 1) : (kt + AHEAD)) * BK * 2;
-#pragma unroll
-        for (int kk = 0; kk < KSTEPS; ++kk) {
-            const int fb = (kk & 1), nb = fb ^ 1;  // KSTEPS is even: step 0 always uses frag[0]
-            const bool last = (kk + 1 == KSTEPS);
-            if (last && NEXT) {
-                if (ISSUE)
+        const unsigned char *a_src = a_base + kbyte, *b_src = b_base + kbyte;
+        const uint32_t dst = cp_lds + fill * Cfg::STAGE_BYTES;
+        static_for<KSTEPS>([&](auto kk_c) {
+            constexpr int kk = decltype(kk_c)::value;
+            constexpr int fb = kk & 1, nb = fb ^ 1;  // an even number of steps: step 0 always uses buffer 0
+            constexpr bool last = (kk + 1 == KSTEPS);
+            if constexpr (last && NEXT) {
+                if constexpr (ISSUE)
                     wait_vmcnt<STEADY_VMCNT>();
                 else
                     wait_vmcnt<0>();
-                if (Cfg::DBG < 3) __syncthreads();
-                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_barrier();
             }
-#pragma unroll
-            for (int idx = 0; idx < NMMA; ++idx) {
-                mma_one(idx, frag[fb]);
-                if (idx < NFRAG && Cfg::DBG < 4) {
-                    if (!last)
-                        read_one(idx, cur, kk + 1, frag[nb]);
-                    else if (NEXT)
-                        read_one(idx, nxt, 0, frag[nb]);
+            __builtin_amdgcn_sched_barrier(0);
+            // Where the operands of the following step come from: the next step of this
+            // chunk, or step 0 of the next chunk (none after the final chunk).
+            constexpr bool prefetch = !last || NEXT;
+            const uint32_t src_bytes = (uint32_t)((last ? nxt : cur) * Cfg::STAGE_BYTES);
+            using SrcKK = std::integral_constant<int, (last ? 0 : kk + 1)>;
+            static_for<NMMA>([&](auto idx_c) {
+                constexpr int idx = decltype(idx_c)::value;
+                mma_one(idx_c, std::integral_constant<int, fb>{});
+                if constexpr (prefetch && Cfg::DBG != 4) {
+                    // A tile t for the next step at slot 2t+1, the double-buffered trailing B
+                    // tiles at slots 2 and 4, leading B tile j in place right after its last use.
+                    if constexpr (idx % 2 == 1 && idx / 2 < TM)
+                        a_frag[nb][idx / 2] = read_a(std::integral_constant<int, idx / 2>{}, src_bytes, SrcKK{});
+                    if constexpr (idx % 2 == 0 && idx >= 2 && idx / 2 - 1 < NDB)
+                        b_last[nb][idx / 2 - 1] =
+                            read_b(std::integral_constant<int, NSB + idx / 2 - 1>{}, src_bytes, SrcKK{});
+                    if constexpr (idx % TM == 0 && idx > 0 && idx / TM - 1 < NSB)
+                        b_frag[idx / TM - 1] = read_b(std::integral_constant<int, idx / TM - 1>{}, src_bytes, SrcKK{});
                 }
-                if (ISSUE && (Cfg::DBG == 0 || Cfg::DBG == 2 || Cfg::DBG == 7)) {
-                    const int slot = kk * NMMA + idx - FIRST_SLOT;  // slot of this MFMA in the copy window
-#pragma unroll
-                    for (int d = 0; d < L; ++d)
-                        if (slot >= 0 && d * SLOTS / L == slot) dma_one(d, kbyte, fill);
+                constexpr int slot = kk * NMMA + idx - FIRST_SLOT;  // slot of this MFMA in the copy window
+                if constexpr (ISSUE && Cfg::DBG != 1 && Cfg::DBG != 4 && slot >= 0) {
+                    // copy instruction d belongs to slot floor(d * SLOTS / L)
+                    constexpr int first = (slot * L + SLOTS - 1) / SLOTS;
+                    constexpr int end = ((slot + 1) * L + SLOTS - 1) / SLOTS;
+                    static_for<end - first>([&](auto d_c) {
+                        dma_one(std::integral_constant<int, first + decltype(d_c)::value>{}, a_src, b_src, dst);
+                    });
                 }
                 __builtin_amdgcn_sched_barrier(0);
-            }
-        }
+            });
+            // Every operand read issued during this step has landed before control leaves
+            // it.  The wait sits here, not at the top of the next step, so that no register
+            // copy the compiler may place on a loop edge can see a fragment in flight.
+            if constexpr (prefetch && Cfg::DBG != 4) wait_operands(std::integral_constant<int, nb>{});
+        });
     };
-    if (Cfg::DBG == 7) {
+    if (trace) {
         t_loop = wall_clock64();
         c_loop = clock64();
     }
@@ -210,14 +399,22 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     }
     iteration(kt, cur, fill, F{}, F{});
 
+    // The MFMAs were issued from assembly, so the compiler neither knows their latency nor
+    // sees any reason to keep its own accumulator reads behind them.  Let the last results
+    // land, then pass every accumulator through an (empty) ordered statement: reads of the
+    // accumulators cannot be scheduled above it.
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    static_for<TM>([&](auto i_c) {
+        static_for<TN>([&](auto j_c) { pin_accumulator(acc[decltype(i_c)::value][decltype(j_c)::value]); });
+    });
     // ---- epilogue: accumulators -> fp16 -> C (through LDS, whole lines per store)
-    if (Cfg::DBG == 7) {
+    if (trace) {
         t_epi = wall_clock64();
         c_epi = clock64();
     }
     __syncthreads();
-    store_tile_via_lds<Cfg>(acc, lds, C, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN, wave, lane);
-    if (Cfg::DBG == 7 && trace && tid == 0) {
+    store_wave_tile<Cfg, Acc>(acc, lds, C, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN, wave, lane);
+    if (trace && tid == 0) {
         __builtin_amdgcn_s_waitcnt(0);
         long long *t = trace + (size_t)blockIdx.x * 8;
         t[0] = t_begin;
