@@ -78,12 +78,16 @@ def _cpu_baseline(torch, A, B, C, budget_s=12.0):
 
 
 def _traffic_bytes():
-    """HBM bytes per launch of the dominant kernel from the committed rocprofv3 counter runs
-    (profiles/), or None when they have not been collected."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic_8192.json")
-    if os.path.exists(path):
+    """Bytes per launch of the dominant kernel between L2 and the memory fabric, from the
+    committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary under profiles/ (None if absent)."""
+    path = os.path.join(ROOT, "profiles", "hgemm_pipelined_256x256x64_square8192_hbm_traffic.txt")
+    try:
         with open(path) as f:
-            return json.load(f).get("traffic_bytes_per_launch")
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":")[1])
+    except OSError:
+        pass
     return None
 
 

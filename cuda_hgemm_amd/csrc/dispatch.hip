@@ -67,8 +67,9 @@ using Skinny64 = SkinnyConfig<64, 128, 2, 2, 4>;
 using Skinny128 = SkinnyConfig<128, 128, 2, 2, 4>;
 using Split64 = SkinnyConfig<64, 64, 2, 2, 4>;
 
-using Big256 = PipeConfig<256, 256, 64, 2, 2, 2>;
-using Mid128 = PipeConfig<128, 128, 64, 2, 2, 3>;
+// 256x256x64 tile on v_mfma_f32_16x16x32_f16, two B buffers and three A buffers (all 160 KB of LDS)
+using Big256 = PipeConfig<256, 256, 64, 2, 2, 2, 16, 8, 0, 1>;
+using Mid128 = PipeConfig<128, 128, 64, 2, 2, 3, 16>;
 
 // Number of K slices for a launch of `tiles` workgroups when `slots` can be resident at
 // once: the power of two (<= 16) that fills the most slots per round; fewer slices win
@@ -170,7 +171,7 @@ extern "C" int hgemm_auto_plan(size_t M, size_t N, size_t K, int *splits) {
 }
 extern "C" const char *hgemm_kernel_name(int kernel) {
     switch (kernel) {
-        case KERNEL_BIG256: return "pipelined 256x256x64, 4 waves, 2-stage ring";
+        case KERNEL_BIG256: return "pipelined 256x256x64, 4 waves, LDS ring 3 (A) + 2 (B)";
         case KERNEL_MID128: return "pipelined 128x128x64, 4 waves, 3-stage ring";
         case KERNEL_SKINNY32: return "split-K 32x128x64, 4-stage ring";
         case KERNEL_SKINNY64: return "split-K 64x128x64, 4-stage ring";

@@ -22,7 +22,7 @@
 namespace hgemm {
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int MI_ = 16, int GROUP_N_ = 8,
-          int DBG_ = 0>
+          int DBG_ = 0, int EXTRA_A_ = 0>
 struct PipeConfig : TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true, GROUP_N_> {
     using Base = TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true, GROUP_N_>;
     // MFMA shape: 32 -> v_mfma_f32_32x32x16_f16, 16 -> v_mfma_f32_16x16x32_f16.  Both move
@@ -38,6 +38,16 @@ struct PipeConfig : TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_
     // 4 = no operand reads in the loop.  (Per-workgroup timestamps are written whenever the
     // launcher is given a trace buffer.)
     static constexpr int DBG = DBG_;
+    // Ring depths.  The B ring has STAGES buffers, the A ring STAGES + EXTRA_A: 256x256x64
+    // tiles are 32 KB per operand and chunk, so the 160 KB of LDS hold two full stages plus
+    // one more A buffer -- the A copies then run two chunks ahead and only the B copies
+    // are on the critical path of the barrier.
+    static constexpr int SA = STAGES_ + EXTRA_A_, SB = STAGES_;
+    static constexpr int RING_BYTES = SA * Base::A_BYTES + SB * Base::B_BYTES;
+    static constexpr int LDS_BYTES =
+        RING_BYTES > Base::WAVES * Base::C_STRIP_BYTES ? RING_BYTES : Base::WAVES * Base::C_STRIP_BYTES;
+    static_assert(EXTRA_A_ == 0 || (EXTRA_A_ == 1 && STAGES_ == 2), "the deeper A ring is defined for two B buffers");
+    static_assert(LDS_BYTES <= 160 * 1024, "exceeds the 160 KB LDS of a gfx950 CU");
     static_assert(MI == 16 || MI == 32, "MFMA tile is 16x16x32 or 32x32x16");
     static_assert(STAGES_ >= 2, "the rotated pipeline needs at least two LDS buffers");
     static_assert(Base::WM % MI == 0 && Base::WN % MI == 0, "wave tile must be a multiple of the MFMA tile");
@@ -165,7 +175,8 @@ __global__ void __launch_bounds__(Cfg::THREADS)
                            int N, int K, int tiles_m, int tiles_n, long long *trace) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
     constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS, CPR = Cfg::CPR, CPS = Cfg::CPS;
-    constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES;
+    constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES, SA = Cfg::SA, SB = Cfg::SB;
+    constexpr int A_BYTES = Cfg::A_BYTES, B_BYTES = Cfg::B_BYTES, B_REGION = SA * A_BYTES;
     constexpr int A_DMA = Cfg::A_DMA, B_DMA = Cfg::B_DMA, L = A_DMA + B_DMA;
     constexpr int NFRAG = TM + TN, NMMA = TM * TN;
     typedef typename MfmaOp<MI>::Acc Acc;
@@ -203,13 +214,16 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     }
     const uint32_t cp_lds = lds_base + wave * 1024;
     // copy instruction `idx` (0..L-1) of chunk at byte offset kbyte into ring buffer `stage`
-    // `a_src` / `b_src` already point at the chunk; `dst` is cp_lds + stage * STAGE_BYTES
-    auto dma_one = [&](auto idx_c, const unsigned char *a_src, const unsigned char *b_src, uint32_t dst) {
+    // LDS is laid out as the A ring (SA buffers) followed by the B ring (SB buffers).
+    // `a_src` / `b_src` already point at the chunk; `dst_a` / `dst_b` are cp_lds plus the
+    // byte offset of the ring buffer to fill.
+    auto dma_one = [&](auto idx_c, const unsigned char *a_src, const unsigned char *b_src, uint32_t dst_a,
+                       uint32_t dst_b) {
         constexpr int idx = decltype(idx_c)::value;
         if constexpr (idx < A_DMA)
-            dma_load16_sv<idx * Cfg::WAVES * 1024>(a_src, voff[idx], dst);
+            dma_load16_sv<idx * Cfg::WAVES * 1024>(a_src, voff[idx], dst_a);
         else
-            dma_load16_sv<Cfg::A_BYTES + (idx - A_DMA) * Cfg::WAVES * 1024>(b_src, voff[idx], dst);
+            dma_load16_sv<(idx - A_DMA) * Cfg::WAVES * 1024>(b_src, voff[idx], dst_b);
     };
 
     // ---- operand fragment set-up: lane l supplies 8 consecutive k (chunk l / MI of the
@@ -217,7 +231,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     const int frag_row = lane % MI;
     const int frag_x = (lane / MI) ^ swizzle_of_row<Cfg>(frag_row);
     const uint32_t a_frag_off = (wm * Cfg::WM + frag_row) * ROW_BYTES;
-    const uint32_t b_frag_off = Cfg::A_BYTES + (wn * Cfg::WN + frag_row) * ROW_BYTES;
+    const uint32_t b_frag_off = B_REGION + (wn * Cfg::WN + frag_row) * ROW_BYTES;
     // Fragment idx sits idx * MI rows further down.  That never changes bits 0-2 of the
     // row's bank-line index, and changes bit 3 (which the swizzle folds into bit 0) only
     // when MI rows are 8 lines: then odd fragments use the chunk index XOR 1.
@@ -249,7 +263,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             a_addr[kk][f] = lds_base + a_frag_off + chunk_off[kk][f];
             b_addr[kk][f] = lds_base + b_frag_off + chunk_off[kk][f];
         }
-    static_assert(Cfg::A_BYTES + (TN - 1) * MI * ROW_BYTES < 65536 && (TM - 1) * MI * ROW_BYTES < 65536,
+    static_assert((TN - 1) * MI * ROW_BYTES < 65536 && (TM - 1) * MI * ROW_BYTES < 65536,
                   "fragment offsets must fit the 16-bit ds_read offset field");
     auto read_a = [&](auto t_c, uint32_t stage_bytes, auto kk_c) -> half8 {
         constexpr int t = decltype(t_c)::value, kk = decltype(kk_c)::value;
@@ -288,27 +302,41 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             MfmaOp<MI>::run(b_frag[j], a_frag[fb][i], acc[i][j]);
     };
 
-    // ---- pipeline.  Chunk c lives in ring buffer c % STAGES.
-    // SPREAD (three or more buffers): the copy of chunk kt+STAGES-1 goes into the buffer
-    // that the barrier of iteration kt-1 released and is issued one instruction at a time
-    // across all MFMA slots of iteration kt, so the texture path sees an even stream.
-    // Otherwise (two buffers): the buffer is only released by this iteration's barrier,
-    // so the copy of chunk kt+STAGES is issued across the slots of the last step.
+    // ---- pipeline.  Chunk c of A lives in A-ring buffer c % SA, of B in B-ring buffer c % SB.
+    // Where the copies of an iteration go (one MFMA "slot" = one MFMA issue):
+    //  SPREAD (three or more buffers each): chunk kt+STAGES-1 goes into the buffers that the
+    //    barrier of iteration kt-1 released, one instruction at a time across all slots.
+    //  DEEP_A (two B buffers, three A buffers): A of chunk kt+2 goes into the A buffer the
+    //    previous barrier released, across the slots of the steps before the last one; B of
+    //    chunk kt+2 goes into the B buffer this iteration's barrier releases, in the first
+    //    half of the last step.  At the next barrier only the B copies are recent.
+    //  otherwise (two buffers each): both operands of chunk kt+2 follow this iteration's
+    //    barrier, across the slots of the last step.
     constexpr bool SPREAD = STAGES >= 3;
-    constexpr int AHEAD = SPREAD ? STAGES - 1 : STAGES;      // chunk kt+AHEAD is copied in iteration kt
-    constexpr int SLOTS = SPREAD ? KSTEPS * NMMA : NMMA;     // MFMA slots the copy is spread over
-    constexpr int FIRST_SLOT = SPREAD ? 0 : (KSTEPS - 1) * NMMA;
+    constexpr bool DEEP_A = (SA == 3 && SB == 2);
+    constexpr int AHEAD = SPREAD ? STAGES - 1 : 2;  // chunk kt+AHEAD is copied in iteration kt
+    constexpr int LAST0 = (KSTEPS - 1) * NMMA;      // first slot of the last step
     static_assert(TM >= 4 && TN >= 2, "the operand schedule needs at least 4 x 2 MFMA tiles per wave");
-    // copy instructions of the current iteration already issued when its barrier is reached
-    constexpr int D_BEFORE = SPREAD ? ((KSTEPS - 1) * NMMA * L + SLOTS - 1) / SLOTS : 0;
+    // slot (0 .. KSTEPS*NMMA-1) in which copy instruction d is issued
+    auto copy_slot = [](int d) constexpr -> int {
+        if (SPREAD) return d * (KSTEPS * NMMA) / L;
+        if (DEEP_A) return d < A_DMA ? d * LAST0 / A_DMA : LAST0 + (d - A_DMA) * (NMMA / 2) / B_DMA;
+        return LAST0 + d * NMMA / L;
+    };
+    // copies of this iteration issued before its barrier (the barrier opens the last step)
+    constexpr int D_BEFORE = SPREAD ? (LAST0 * L + KSTEPS * NMMA - 1) / (KSTEPS * NMMA) : (DEEP_A ? A_DMA : 0);
     // copies allowed to be still in flight at the barrier while chunk kt+1 must have landed
-    constexpr int STEADY_VMCNT = SPREAD ? (STAGES - 3) * L + D_BEFORE : (STAGES - 2) * L;
+    constexpr int STEADY_VMCNT = SPREAD ? (STAGES - 3) * L + D_BEFORE : D_BEFORE;
     static_assert(STEADY_VMCNT <= 63, "vmcnt is a 6-bit counter");
+    // ring buffer (relative to the current one) that this iteration's copies fill
+    constexpr int FILL_OFF_A = SPREAD ? SA - 1 : (DEEP_A ? 2 : 0);
+    constexpr int FILL_OFF_B = SPREAD ? SB - 1 : 0;
 
     static_for<AHEAD>([&](auto s_c) {
         constexpr int st = decltype(s_c)::value;
         static_for<L>([&](auto idx_c) {
-            dma_one(idx_c, a_base + st * BK * 2, b_base + st * BK * 2, cp_lds + st * Cfg::STAGE_BYTES);
+            dma_one(idx_c, a_base + st * BK * 2, b_base + st * BK * 2, cp_lds + st * A_BYTES,
+                    cp_lds + B_REGION + st * B_BYTES);
         });
     });
     wait_vmcnt<(AHEAD - 1) * L>();
@@ -323,12 +351,14 @@ __global__ void __launch_bounds__(Cfg::THREADS)
 
     // One iteration = one K chunk.  ISSUE: chunk kt+AHEAD exists and is copied now.
     // NEXT: chunk kt+1 exists (the barrier is needed and its operands are prefetched).
-    auto iteration = [&](int kt, int cur, int fill, auto issue_tag, auto next_tag) {
+    auto iteration = [&](int kt, int cur_a, int cur_b, auto issue_tag, auto next_tag) {
         constexpr bool ISSUE = decltype(issue_tag)::value, NEXT = decltype(next_tag)::value;
-        const int nxt = (cur + 1 == STAGES) ? 0 : cur + 1;
+        const int nxt_a = (cur_a + 1 == SA) ? 0 : cur_a + 1;
+        const int nxt_b = (cur_b + 1 == SB) ? 0 : cur_b + 1;
+        const int fill_a = (cur_a + FILL_OFF_A) % SA, fill_b = (cur_b + FILL_OFF_B) % SB;
         const int kbyte = (Cfg::DBG == 2 ? (kt & 1) : (kt + AHEAD)) * BK * 2;
         const unsigned char *a_src = a_base + kbyte, *b_src = b_base + kbyte;
-        const uint32_t dst = cp_lds + fill * Cfg::STAGE_BYTES;
+        const uint32_t dst_a = cp_lds + fill_a * A_BYTES, dst_b = cp_lds + B_REGION + fill_b * B_BYTES;
         static_for<KSTEPS>([&](auto kk_c) {
             constexpr int kk = decltype(kk_c)::value;
             constexpr int fb = kk & 1, nb = fb ^ 1;  // an even number of steps: step 0 always uses buffer 0
@@ -344,7 +374,8 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             // Where the operands of the following step come from: the next step of this
             // chunk, or step 0 of the next chunk (none after the final chunk).
             constexpr bool prefetch = !last || NEXT;
-            const uint32_t src_bytes = (uint32_t)((last ? nxt : cur) * Cfg::STAGE_BYTES);
+            const uint32_t src_a = (uint32_t)((last ? nxt_a : cur_a) * A_BYTES);
+            const uint32_t src_b = (uint32_t)((last ? nxt_b : cur_b) * B_BYTES);
             using SrcKK = std::integral_constant<int, (last ? 0 : kk + 1)>;
             static_for<NMMA>([&](auto idx_c) {
                 constexpr int idx = decltype(idx_c)::value;
@@ -353,20 +384,17 @@ __global__ void __launch_bounds__(Cfg::THREADS)
                     // A tile t for the next step at slot 2t+1, the double-buffered trailing B
                     // tiles at slots 2 and 4, leading B tile j in place right after its last use.
                     if constexpr (idx % 2 == 1 && idx / 2 < TM)
-                        a_frag[nb][idx / 2] = read_a(std::integral_constant<int, idx / 2>{}, src_bytes, SrcKK{});
+                        a_frag[nb][idx / 2] = read_a(std::integral_constant<int, idx / 2>{}, src_a, SrcKK{});
                     if constexpr (idx % 2 == 0 && idx >= 2 && idx / 2 - 1 < NDB)
                         b_last[nb][idx / 2 - 1] =
-                            read_b(std::integral_constant<int, NSB + idx / 2 - 1>{}, src_bytes, SrcKK{});
+                            read_b(std::integral_constant<int, NSB + idx / 2 - 1>{}, src_b, SrcKK{});
                     if constexpr (idx % TM == 0 && idx > 0 && idx / TM - 1 < NSB)
-                        b_frag[idx / TM - 1] = read_b(std::integral_constant<int, idx / TM - 1>{}, src_bytes, SrcKK{});
+                        b_frag[idx / TM - 1] = read_b(std::integral_constant<int, idx / TM - 1>{}, src_b, SrcKK{});
                 }
-                constexpr int slot = kk * NMMA + idx - FIRST_SLOT;  // slot of this MFMA in the copy window
-                if constexpr (ISSUE && Cfg::DBG != 1 && Cfg::DBG != 4 && slot >= 0) {
-                    // copy instruction d belongs to slot floor(d * SLOTS / L)
-                    constexpr int first = (slot * L + SLOTS - 1) / SLOTS;
-                    constexpr int end = ((slot + 1) * L + SLOTS - 1) / SLOTS;
-                    static_for<end - first>([&](auto d_c) {
-                        dma_one(std::integral_constant<int, first + decltype(d_c)::value>{}, a_src, b_src, dst);
+                if constexpr (ISSUE && Cfg::DBG != 1 && Cfg::DBG != 4) {
+                    static_for<L>([&](auto d_c) {
+                        if constexpr (copy_slot(decltype(d_c)::value) == kk * NMMA + idx)
+                            dma_one(d_c, a_src, b_src, dst_a, dst_b);
                     });
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -384,20 +412,20 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     using T = std::true_type;
     using F = std::false_type;
 
-    int kt = 0, cur = 0, fill = SPREAD ? STAGES - 1 : 0;
+    int kt = 0, cur_a = 0, cur_b = 0;
     auto advance = [&] {
-        cur = (cur + 1 == STAGES) ? 0 : cur + 1;
-        fill = (fill + 1 == STAGES) ? 0 : fill + 1;
+        cur_a = (cur_a + 1 == SA) ? 0 : cur_a + 1;
+        cur_b = (cur_b + 1 == SB) ? 0 : cur_b + 1;
     };
     for (; kt < num_k - AHEAD; ++kt) {  // chunk kt+AHEAD exists
-        iteration(kt, cur, fill, T{}, T{});
+        iteration(kt, cur_a, cur_b, T{}, T{});
         advance();
     }
     for (; kt < num_k - 1; ++kt) {  // drain: nothing left to copy
-        iteration(kt, cur, fill, F{}, T{});
+        iteration(kt, cur_a, cur_b, F{}, T{});
         advance();
     }
-    iteration(kt, cur, fill, F{}, F{});
+    iteration(kt, cur_a, cur_b, F{}, F{});
 
     // The MFMAs were issued from assembly, so the compiler neither knows their latency nor
     // sees any reason to keep its own accumulator reads behind them.  Let the last results
@@ -433,7 +461,7 @@ void launch_pipelined(const void *A, const void *B, void *C, size_t M, size_t N,
     check_operands(A, B, C, M, N, K);
     HGEMM_CHECK_MSG(Cfg::supports(M, N, K),
                     "%s needs M %% %d == 0, N %% %d == 0, K %% %d == 0, K >= %d (got M=%zu N=%zu K=%zu)", name,
-                    Cfg::BM, Cfg::BN, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
+                    Cfg::BM, Cfg::BN, Cfg::BK, Cfg::BK * (Cfg::SA + 1), M, N, K);
     static bool configured = [] {
         HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
