@@ -61,67 +61,71 @@ void launch_splitk(const void *A, const void *B, void *C, size_t M, size_t N, si
     }
 }
 
-//                         BM   BN  WM WN stages
-using Skinny32 = SkinnyConfig<32, 128, 1, 4, 4>;
-using Skinny64 = SkinnyConfig<64, 128, 2, 2, 4>;
-using Skinny128 = SkinnyConfig<128, 128, 2, 2, 4>;
-using Split64 = SkinnyConfig<64, 64, 2, 2, 4>;
+//                             BM   BN  WM WN stages
+using Split32x64 = SkinnyConfig<32, 64, 1, 2, 4>;
+using Split64x64 = SkinnyConfig<64, 64, 2, 2, 4>;
+using Split64x128 = SkinnyConfig<64, 128, 2, 2, 4>;
+using Split128x64 = SkinnyConfig<128, 64, 2, 2, 4>;
+using Split128x128 = SkinnyConfig<128, 128, 2, 2, 4>;
 
 // 256x256x64 tile on v_mfma_f32_16x16x32_f16, two B buffers and three A buffers (all 160 KB of LDS)
 using Big256 = PipeConfig<256, 256, 64, 2, 2, 2, 16, 8, 0, 1>;
-using Mid128 = PipeConfig<128, 128, 64, 2, 2, 3, 16>;
+using Mid128 = PipeConfig<128, 128, 64, 2, 2, 5, 16>;
+using Mid128S4 = PipeConfig<128, 128, 64, 2, 2, 4, 16>;
+using Small64 = PipeConfig<64, 64, 64, 1, 1, 3, 16>;
 
-// Number of K slices for a launch of `tiles` workgroups when `slots` can be resident at
-// once: the power of two (<= 16) that fills the most slots per round; fewer slices win
-// ties.  Each slice must be a whole number of 64-wide chunks and at least two of them.
-int choose_splits(size_t tiles, size_t slots, size_t K) {
-    int best = 1;
-    double best_fill = 0.0;
-    for (int s = 1; s <= 16; s *= 2) {
-        if (K % ((size_t)s * 64) != 0 || K / s < 128) break;
-        const size_t wgs = tiles * s;
-        const size_t rounds = div_ceil(wgs, slots);
-        const double fill = (double)wgs / (double)(rounds * slots);
-        if (fill > best_fill + 0.02) {
-            best_fill = fill;
-            best = s;
-        }
-    }
-    return best;
+// Number of K slices for `tiles` output tiles: the smallest power of two (<= 16) that
+// gives at least three quarters of the CUs a workgroup.  Each slice is a whole number of 64-wide chunks, at least
+// two of them.  (Measured on the decode shapes: more slices than that only add partial-sum
+// traffic, fewer leave CUs without a stream of B.)
+int choose_splits(size_t tiles, size_t cus, size_t K) {
+    int s = 1;
+    while (s < 16 && tiles * s < cus * 3 / 4 && K % ((size_t)s * 2 * 64) == 0 && K / (s * 2) >= 128) s *= 2;
+    return s;
 }
 
 }  // namespace
 
 bool skinny_supports(size_t M, size_t N, size_t K) {
-    return M >= 1 && M <= 128 && N % 128 == 0 && K % 64 == 0 && N > 0 && K > 0;
+    return M >= 1 && M <= 128 && N > 0 && N % 64 == 0 && K > 0 && K % 64 == 0;
 }
 
+// Choices below come from timing every candidate (tile x slices) on the specification's
+// shapes on an MI355X, operands rotated so small problems read HBM.
 Plan plan_for(size_t M, size_t N, size_t K) {
     Plan p;
     if (M == 0 || N == 0 || K == 0) return p;
     const size_t cus = (size_t)compute_units();
     if (skinny_supports(M, N, K)) {
-        p.kernel = M <= 32 ? KERNEL_SKINNY32 : (M <= 64 ? KERNEL_SKINNY64 : KERNEL_SKINNY128);
-        const size_t per_cu = M <= 32 ? 2 : 1;  // ring of 80 KB fits twice in 160 KB of LDS
-        p.splits = choose_splits(N / 128, cus * per_cu, K);
+        if (M == 128 && N >= 8192 && N % 128 == 0 && Mid128S4::supports(M, N, K)) {
+            p.kernel = KERNEL_MID128_S4;
+            return p;
+        }
+        const bool wide = M > 32 && N >= 16384 && N % 128 == 0;  // enough columns: 128-wide tiles stream B better
+        if (M <= 32)
+            p.kernel = KERNEL_SPLIT_32x64;
+        else if (M <= 64)
+            p.kernel = wide ? KERNEL_SPLIT_64x128 : KERNEL_SPLIT_64x64;
+        else
+            p.kernel = wide ? KERNEL_SPLIT_128x128 : KERNEL_SPLIT_128x64;
+        p.splits = choose_splits(N / (wide ? 128 : 64), cus, K);
         return p;
     }
     if (Big256::supports(M, N, K) && (M / 256) * (N / 256) >= cus * 3 / 4) {
         p.kernel = KERNEL_BIG256;
         return p;
     }
-    if (Mid128::supports(M, N, K) && (M / 128) * (N / 128) >= cus * 3 / 4) {
+    if (Mid128::supports(M, N, K) && (M / 128) * (N / 128) >= cus * 3 / 8) {
         p.kernel = KERNEL_MID128;
         return p;
     }
-    if (N % 128 == 0 && K % 64 == 0 && (div_ceil(M, 128) * (N / 128)) >= cus / 8) {
-        p.kernel = KERNEL_SPLIT128;
-        p.splits = choose_splits(div_ceil(M, 128) * (N / 128), cus, K);
+    if (Small64::supports(M, N, K)) {
+        p.kernel = KERNEL_SMALL64;
         return p;
     }
-    if (N % 64 == 0 && K % 64 == 0) {
-        p.kernel = KERNEL_SPLIT64;
-        p.splits = choose_splits(div_ceil(M, 64) * (N / 64), cus * 2, K);
+    if (N % 64 == 0 && K % 64 == 0) {  // any M: rows beyond M are guarded
+        p.kernel = KERNEL_SPLIT_64x64;
+        p.splits = choose_splits(div_ceil(M, 64) * (N / 64), cus, K);
         return p;
     }
     p.kernel = KERNEL_SIMT;
@@ -132,11 +136,13 @@ void run_plan(const Plan &p, const void *A, const void *B, void *C, size_t M, si
     switch (p.kernel) {
         case KERNEL_BIG256: launch_pipelined<Big256>(A, B, C, M, N, K, "hgemm_auto"); break;
         case KERNEL_MID128: launch_pipelined<Mid128>(A, B, C, M, N, K, "hgemm_auto"); break;
-        case KERNEL_SKINNY32: launch_splitk<Skinny32>(A, B, C, M, N, K, p.splits); break;
-        case KERNEL_SKINNY64: launch_splitk<Skinny64>(A, B, C, M, N, K, p.splits); break;
-        case KERNEL_SKINNY128:
-        case KERNEL_SPLIT128: launch_splitk<Skinny128>(A, B, C, M, N, K, p.splits); break;
-        case KERNEL_SPLIT64: launch_splitk<Split64>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_MID128_S4: launch_pipelined<Mid128S4>(A, B, C, M, N, K, "hgemm_auto"); break;
+        case KERNEL_SMALL64: launch_pipelined<Small64>(A, B, C, M, N, K, "hgemm_auto"); break;
+        case KERNEL_SPLIT_32x64: launch_splitk<Split32x64>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_SPLIT_64x64: launch_splitk<Split64x64>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_SPLIT_64x128: launch_splitk<Split64x128>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_SPLIT_128x64: launch_splitk<Split128x64>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_SPLIT_128x128: launch_splitk<Split128x128>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_SIMT:
             hgemm_simt_naive(reinterpret_cast<const hgemm_half *>(A), reinterpret_cast<const hgemm_half *>(B),
                              reinterpret_cast<hgemm_half *>(C), M, N, K);
@@ -152,7 +158,7 @@ using namespace hgemm;
 extern "C" void hgemm_skinny(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K) {
     check_operands(A, B, C, M, N, K);
     HGEMM_CHECK_MSG(skinny_supports(M, N, K),
-                    "hgemm_skinny needs M <= 128, N %% 128 == 0, K %% 64 == 0 (got M=%zu N=%zu K=%zu)", M, N, K);
+                    "hgemm_skinny needs M <= 128, N %% 64 == 0, K %% 64 == 0 (got M=%zu N=%zu K=%zu)", M, N, K);
     run_plan(plan_for(M, N, K), A, B, C, M, N, K);
 }
 extern "C" int hgemm_skinny_supports(size_t M, size_t N, size_t K) { return skinny_supports(M, N, K) ? 1 : 0; }
@@ -172,12 +178,14 @@ extern "C" int hgemm_auto_plan(size_t M, size_t N, size_t K, int *splits) {
 extern "C" const char *hgemm_kernel_name(int kernel) {
     switch (kernel) {
         case KERNEL_BIG256: return "pipelined 256x256x64, 4 waves, LDS ring 3 (A) + 2 (B)";
-        case KERNEL_MID128: return "pipelined 128x128x64, 4 waves, 3-stage ring";
-        case KERNEL_SKINNY32: return "split-K 32x128x64, 4-stage ring";
-        case KERNEL_SKINNY64: return "split-K 64x128x64, 4-stage ring";
-        case KERNEL_SKINNY128: return "split-K 128x128x64, 4-stage ring";
-        case KERNEL_SPLIT128: return "split-K 128x128x64, 4-stage ring";
-        case KERNEL_SPLIT64: return "split-K 64x64x64, 4-stage ring";
+        case KERNEL_MID128: return "pipelined 128x128x64, 4 waves, 5-stage ring";
+        case KERNEL_MID128_S4: return "pipelined 128x128x64, 4 waves, 4-stage ring";
+        case KERNEL_SMALL64: return "pipelined 64x64x64, 1 wave, 3-stage ring";
+        case KERNEL_SPLIT_32x64: return "split-K 32x64x64, 2 waves, 4-stage ring";
+        case KERNEL_SPLIT_64x64: return "split-K 64x64x64, 4 waves, 4-stage ring";
+        case KERNEL_SPLIT_64x128: return "split-K 64x128x64, 4 waves, 4-stage ring";
+        case KERNEL_SPLIT_128x64: return "split-K 128x64x64, 4 waves, 4-stage ring";
+        case KERNEL_SPLIT_128x128: return "split-K 128x128x64, 4 waves, 4-stage ring";
         case KERNEL_SIMT: return "scalar fallback";
         default: return "none";
     }

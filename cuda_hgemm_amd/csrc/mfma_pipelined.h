@@ -203,14 +203,21 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     constexpr int DMA_ROW_STEP = Cfg::WAVES * Cfg::ROWS_PER_DMA;
     uint32_t voff[L];
     {
-        const int row = wave * Cfg::ROWS_PER_DMA + lane / CPR;
-        const int ch = (lane % CPR) ^ swizzle_of_row<Cfg>(row);
+        // lane l of instruction `it` lands on physical chunk l % CPR of LDS row
+        // row0 + it * DMA_ROW_STEP, so it fetches the logical chunk the swizzle maps there
+        const int row0 = wave * Cfg::ROWS_PER_DMA + lane / CPR;
 #pragma unroll
-        for (int it = 0; it < A_DMA; ++it)
-            voff[it] = ((uint32_t)(row + it * DMA_ROW_STEP) * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
+        for (int it = 0; it < A_DMA; ++it) {
+            const int row = row0 + it * DMA_ROW_STEP;
+            const int ch = (lane % CPR) ^ swizzle_of_row<Cfg>(row);
+            voff[it] = ((uint32_t)row * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
+        }
 #pragma unroll
-        for (int it = 0; it < B_DMA; ++it)
-            voff[A_DMA + it] = ((uint32_t)(row + it * DMA_ROW_STEP) * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
+        for (int it = 0; it < B_DMA; ++it) {
+            const int row = row0 + it * DMA_ROW_STEP;
+            const int ch = (lane % CPR) ^ swizzle_of_row<Cfg>(row);
+            voff[A_DMA + it] = ((uint32_t)row * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
+        }
     }
     const uint32_t cp_lds = lds_base + wave * 1024;
     // copy instruction `idx` (0..L-1) of chunk at byte offset kbyte into ring buffer `stage`

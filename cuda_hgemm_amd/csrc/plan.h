@@ -7,14 +7,16 @@ namespace hgemm {
 
 enum KernelId {
     KERNEL_NONE = 0,
-    KERNEL_BIG256,     // pipelined 256x256x64
-    KERNEL_MID128,     // pipelined 128x128x64
-    KERNEL_SKINNY32,   // M <= 32
-    KERNEL_SKINNY64,   // M <= 64
-    KERNEL_SKINNY128,  // M <= 128
-    KERNEL_SPLIT128,   // 128x128 tiles with K slices (few tiles, long K)
-    KERNEL_SPLIT64,    // 64x64 tiles with K slices
-    KERNEL_SIMT,       // scalar fallback for shapes no MFMA kernel tiles
+    KERNEL_BIG256,      // pipelined 256x256x64, 4 waves
+    KERNEL_MID128,      // pipelined 128x128x64, 4 waves, 5-stage ring
+    KERNEL_MID128_S4,   // pipelined 128x128x64, 4 waves, 4-stage ring (M = 128 against a very wide B)
+    KERNEL_SMALL64,     // pipelined 64x64x64, 1 wave, 3-stage ring
+    KERNEL_SPLIT_32x64,   // split-K family: BM x BN tile, 4-stage ring, M guarded
+    KERNEL_SPLIT_64x64,
+    KERNEL_SPLIT_64x128,
+    KERNEL_SPLIT_128x64,
+    KERNEL_SPLIT_128x128,
+    KERNEL_SIMT,        // scalar fallback for shapes no MFMA kernel tiles
 };
 
 struct Plan {

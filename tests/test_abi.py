@@ -69,7 +69,7 @@ def test_shape_predicates(hgemm_lib):
         assert not s(name, 128, 128, 256) and not s(name, 256, 64, 256) and not s(name, 256, 128, 48)
     assert not s("hgemm_mfma_async_stage4", 256, 128, 64)      # K must cover the 3-chunk prologue
     assert s("hgemm_mfma_async_stage4", 256, 128, 96)
-    assert s("hgemm_skinny", 1, 4096, 4096) and s("hgemm_skinny", 128, 28672, 4096)
+    assert s("hgemm_skinny", 1, 4096, 4096) and s("hgemm_skinny", 128, 28672, 4096) and s("hgemm_skinny", 8, 192, 64)
     assert not s("hgemm_skinny", 129, 4096, 4096) and not s("hgemm_skinny", 8, 100, 4096)
     assert not s("hgemm_auto", 0, 8, 8) and not s("hgemm_auto", 1 << 20, 8, 1 << 20)
 
@@ -85,7 +85,7 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
     for m in (1, 8, 16, 64, 128):
         for n in (4096, 28672):
             p = plan(m, n, 4096)
-            assert p["kernel"].startswith("split-K"), (m, n, p)
+            assert p["kernel"].startswith("split-K") or (m == 128 and p["kernel"].startswith("pipelined 128x128")), (m, n, p)
             assert 4096 % (p["splits"] * 64) == 0
     assert plan(100, 100, 100)["kernel"] == "scalar fallback"
 
