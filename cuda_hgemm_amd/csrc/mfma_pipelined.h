@@ -315,8 +315,8 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     //    barrier of iteration kt-1 released, one instruction at a time across all slots.
     //  DEEP_A (two B buffers, three A buffers): A of chunk kt+2 goes into the A buffer the
     //    previous barrier released, across the slots of the steps before the last one; B of
-    //    chunk kt+2 goes into the B buffer this iteration's barrier releases, in the first
-    //    half of the last step.  At the next barrier only the B copies are recent.
+    //    chunk kt+2 goes into the B buffer this iteration's barrier releases, across the
+    //    slots of the last step.  At the next barrier only the B copies are recent.
     //  otherwise (two buffers each): both operands of chunk kt+2 follow this iteration's
     //    barrier, across the slots of the last step.
     constexpr bool SPREAD = STAGES >= 3;
@@ -324,10 +324,14 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     constexpr int AHEAD = SPREAD ? STAGES - 1 : 2;  // chunk kt+AHEAD is copied in iteration kt
     constexpr int LAST0 = (KSTEPS - 1) * NMMA;      // first slot of the last step
     static_assert(TM >= 4 && TN >= 2, "the operand schedule needs at least 4 x 2 MFMA tiles per wave");
-    // slot (0 .. KSTEPS*NMMA-1) in which copy instruction d is issued
+    // Slot (0 .. KSTEPS*NMMA-1) in which copy instruction d is issued.  Copies are spread
+    // evenly and sit in odd slots (operand reads use even ones): issuing them closer
+    // together is slower, and staggering the waves of a workgroup against each other was
+    // measured and makes no difference.
     auto copy_slot = [](int d) constexpr -> int {
         if (SPREAD) return d * (KSTEPS * NMMA) / L;
-        if (DEEP_A) return d < A_DMA ? d * LAST0 / A_DMA : LAST0 + (d - A_DMA) * (NMMA / 2) / B_DMA;
+        if (DEEP_A)
+            return d < A_DMA ? d * LAST0 / A_DMA + 5 : LAST0 + (d - A_DMA) * NMMA / B_DMA + 3;
         return LAST0 + d * NMMA / L;
     };
     // copies of this iteration issued before its barrier (the barrier opens the last step)
@@ -388,15 +392,19 @@ __global__ void __launch_bounds__(Cfg::THREADS)
                 constexpr int idx = decltype(idx_c)::value;
                 mma_one(idx_c, std::integral_constant<int, fb>{});
                 if constexpr (prefetch && Cfg::DBG != 4) {
-                    // A tile t for the next step at slot 2t+1, the double-buffered trailing B
-                    // tiles at slots 2 and 4, leading B tile j in place right after its last use.
-                    if constexpr (idx % 2 == 1 && idx / 2 < TM)
-                        a_frag[nb][idx / 2] = read_a(std::integral_constant<int, idx / 2>{}, src_a, SrcKK{});
-                    if constexpr (idx % 2 == 0 && idx >= 2 && idx / 2 - 1 < NDB)
-                        b_last[nb][idx / 2 - 1] =
-                            read_b(std::integral_constant<int, NSB + idx / 2 - 1>{}, src_b, SrcKK{});
-                    if constexpr (idx % TM == 0 && idx > 0 && idx / TM - 1 < NSB)
-                        b_frag[idx / TM - 1] = read_b(std::integral_constant<int, idx / TM - 1>{}, src_b, SrcKK{});
+                    // One operand read per slot at most, spread out (an LDS read in the slot
+                    // right after another one stalls MFMA issue): A tile t for the next step
+                    // at slot RS*t + 2, the double-buffered trailing B tiles at slots 0 and
+                    // RS, leading B tile j in place RS slots after its last use (TM*j + TM - 1).
+                    constexpr int RS = (NMMA / 2) / TM >= 2 ? (NMMA / 2) / TM : 1;  // 4 for 64 MFMAs, 8 A tiles
+                    if constexpr (idx >= 2 && (idx - 2) % RS == 0 && (idx - 2) / RS < TM)
+                        a_frag[nb][(idx - 2) / RS] =
+                            read_a(std::integral_constant<int, (idx - 2) / RS>{}, src_a, SrcKK{});
+                    if constexpr (idx % RS == 0 && idx / RS < NDB)
+                        b_last[nb][idx / RS] = read_b(std::integral_constant<int, NSB + idx / RS>{}, src_b, SrcKK{});
+                    if constexpr (idx >= TM + RS && (idx - RS) % TM == 0 && (idx - RS) / TM - 1 < NSB)
+                        b_frag[(idx - RS) / TM - 1] =
+                            read_b(std::integral_constant<int, (idx - RS) / TM - 1>{}, src_b, SrcKK{});
                 }
                 if constexpr (ISSUE && Cfg::DBG != 1 && Cfg::DBG != 4) {
                     static_for<L>([&](auto d_c) {
@@ -468,7 +476,7 @@ void launch_pipelined(const void *A, const void *B, void *C, size_t M, size_t N,
     check_operands(A, B, C, M, N, K);
     HGEMM_CHECK_MSG(Cfg::supports(M, N, K),
                     "%s needs M %% %d == 0, N %% %d == 0, K %% %d == 0, K >= %d (got M=%zu N=%zu K=%zu)", name,
-                    Cfg::BM, Cfg::BN, Cfg::BK, Cfg::BK * (Cfg::SA + 1), M, N, K);
+                    Cfg::BM, Cfg::BN, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
     static bool configured = [] {
         HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
