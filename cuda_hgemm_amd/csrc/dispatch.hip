@@ -73,6 +73,57 @@ using Big256 = PipeConfig<256, 256, 64, 2, 2, 2, 16, 8, 0, 1>;
 using Mid128 = PipeConfig<128, 128, 64, 2, 2, 5, 16>;
 using Mid128S4 = PipeConfig<128, 128, 64, 2, 2, 4, 16>;
 using Small64 = PipeConfig<64, 64, 64, 1, 1, 3, 16>;
+using Tile192 = PipeConfig<192, 192, 64, 2, 2, 3, 16>;
+using Rect256x128 = PipeConfig<256, 128, 64, 2, 2, 3, 16>;
+
+// Pipelined kernel with K cut into `splits` slices: fp32 partial sums per slice, then the
+// ordered reduction (the same one the small-M kernel uses), so the result is bit-identical
+// from run to run.
+template <class Cfg>
+void launch_pipelined_plan(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, int splits) {
+    if (splits <= 1) {
+        launch_pipelined<Cfg>(A, B, C, M, N, K, "hgemm_auto");
+        return;
+    }
+    float *partial = splitk_workspace((size_t)splits * M * N * sizeof(float));
+    launch_pipelined_split<Cfg>(A, B, partial, M, N, K, splits, "hgemm_auto");
+    const size_t elems = M * N;  // a multiple of 8: every tile dimension is
+    splitk_reduce_kernel<<<dim3((unsigned)div_ceil(elems / 8, 256)), dim3(256), 0, nullptr>>>(
+        partial, reinterpret_cast<half_t *>(C), elems, splits);
+    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+}
+
+// ---- cost model for the tile-aligned shapes.  A candidate is a tile (its kernel), how
+// many of its workgroups a CU holds, and three times in microseconds fitted to
+// measurements on an MI355X over ~60 shapes (rms error 7 %): `fix` per workgroup
+// (prologue, epilogue, scheduling) and the time of one 64-wide K chunk with few (`lo`)
+// and with all (`hi`) CUs busy -- the chip is power-limited, so a chunk costs more when
+// the whole chip computes.  time = launch + full rounds * (fix + chunks * hi)
+//                                 + last partial round * (fix + chunks * between lo and hi)
+//                                 + reduction of the fp32 partials when K is split.
+struct Candidate {
+    int kernel, bm, bn, per_cu, stages;
+    double fix, lo, hi;
+};
+constexpr Candidate CANDIDATES[] = {
+    {KERNEL_BIG256, 256, 256, 1, 2, 7.02, 0.959, 1.567},
+    {KERNEL_T192, 192, 192, 1, 3, 4.79, 0.585, 1.036},
+    {KERNEL_R256x128, 256, 128, 1, 3, 3.83, 0.561, 0.924},
+    {KERNEL_MID128, 128, 128, 1, 5, 2.99, 0.340, 0.543},
+    {KERNEL_SMALL64, 64, 64, 3, 3, 1.61, 0.394, 0.604},
+};
+constexpr double LAUNCH_US = 0.38, REDUCE_US = 4.86, REDUCE_BYTES_PER_US = 7207e3;
+constexpr size_t MAX_PARTIAL_BYTES = 512ull << 20;
+
+double predict_us(const Candidate &c, size_t M, size_t N, size_t K, int splits, size_t cus) {
+    const size_t wgs = (M / c.bm) * (N / c.bn) * (size_t)splits, slots = cus * (size_t)c.per_cu;
+    const double chunks = (double)(K / (size_t)splits / 64);
+    const size_t full = wgs / slots, rem = wgs % slots;
+    double t = LAUNCH_US + (double)full * (c.fix + chunks * c.hi);
+    if (rem) t += c.fix + chunks * (c.lo + (c.hi - c.lo) * (double)rem / (double)slots);
+    if (splits > 1) t += REDUCE_US + (double)splits * (double)M * (double)N * 8.0 / REDUCE_BYTES_PER_US;
+    return t;
+}
 
 // Number of K slices for `tiles` output tiles: the smallest power of two (<= 16) that
 // gives at least three quarters of the CUs a workgroup.  Each slice is a whole number of 64-wide chunks, at least
@@ -90,8 +141,9 @@ bool skinny_supports(size_t M, size_t N, size_t K) {
     return M >= 1 && M <= 128 && N > 0 && N % 64 == 0 && K > 0 && K % 64 == 0;
 }
 
-// Choices below come from timing every candidate (tile x slices) on the specification's
-// shapes on an MI355X, operands rotated so small problems read HBM.
+// M <= 128: choices come from timing every candidate (tile x slices) on the specification's
+// decode shapes on an MI355X, operands rotated so small problems read HBM.  Larger,
+// tile-aligned shapes: the cheapest (tile, slices) pair under the cost model above.
 Plan plan_for(size_t M, size_t N, size_t K) {
     Plan p;
     if (M == 0 || N == 0 || K == 0) return p;
@@ -111,18 +163,21 @@ Plan plan_for(size_t M, size_t N, size_t K) {
         p.splits = choose_splits(N / (wide ? 128 : 64), cus, K);
         return p;
     }
-    if (Big256::supports(M, N, K) && (M / 256) * (N / 256) >= cus * 3 / 4) {
-        p.kernel = KERNEL_BIG256;
-        return p;
+    double best = 0.0;
+    for (const Candidate &c : CANDIDATES) {
+        if (M % c.bm || N % c.bn) continue;
+        for (int s = 1; s <= 32; s *= 2) {
+            if (K % ((size_t)s * 64) || K / s < (size_t)64 * c.stages) break;
+            if (s > 1 && (size_t)s * M * N * sizeof(float) > MAX_PARTIAL_BYTES) break;
+            const double t = predict_us(c, M, N, K, s, cus);
+            if (p.kernel == KERNEL_NONE || t < best) {
+                best = t;
+                p.kernel = c.kernel;
+                p.splits = s;
+            }
+        }
     }
-    if (Mid128::supports(M, N, K) && (M / 128) * (N / 128) >= cus * 3 / 8) {
-        p.kernel = KERNEL_MID128;
-        return p;
-    }
-    if (Small64::supports(M, N, K)) {
-        p.kernel = KERNEL_SMALL64;
-        return p;
-    }
+    if (p.kernel != KERNEL_NONE) return p;
     if (N % 64 == 0 && K % 64 == 0) {  // any M: rows beyond M are guarded
         p.kernel = KERNEL_SPLIT_64x64;
         p.splits = choose_splits(div_ceil(M, 64) * (N / 64), cus, K);
@@ -134,10 +189,12 @@ Plan plan_for(size_t M, size_t N, size_t K) {
 
 void run_plan(const Plan &p, const void *A, const void *B, void *C, size_t M, size_t N, size_t K) {
     switch (p.kernel) {
-        case KERNEL_BIG256: launch_pipelined<Big256>(A, B, C, M, N, K, "hgemm_auto"); break;
-        case KERNEL_MID128: launch_pipelined<Mid128>(A, B, C, M, N, K, "hgemm_auto"); break;
+        case KERNEL_BIG256: launch_pipelined_plan<Big256>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_T192: launch_pipelined_plan<Tile192>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_R256x128: launch_pipelined_plan<Rect256x128>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_MID128_S4: launch_pipelined<Mid128S4>(A, B, C, M, N, K, "hgemm_auto"); break;
-        case KERNEL_SMALL64: launch_pipelined<Small64>(A, B, C, M, N, K, "hgemm_auto"); break;
+        case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_SPLIT_32x64: launch_splitk<Split32x64>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_SPLIT_64x64: launch_splitk<Split64x64>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_SPLIT_64x128: launch_splitk<Split64x128>(A, B, C, M, N, K, p.splits); break;
@@ -181,6 +238,8 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
         case KERNEL_MID128: return "pipelined 128x128x64, 4 waves, 5-stage ring";
         case KERNEL_MID128_S4: return "pipelined 128x128x64, 4 waves, 4-stage ring";
         case KERNEL_SMALL64: return "pipelined 64x64x64, 1 wave, 3-stage ring";
+        case KERNEL_T192: return "pipelined 192x192x64, 4 waves, 3-stage ring";
+        case KERNEL_R256x128: return "pipelined 256x128x64, 4 waves, 3-stage ring";
         case KERNEL_SPLIT_32x64: return "split-K 32x64x64, 2 waves, 4-stage ring";
         case KERNEL_SPLIT_64x64: return "split-K 64x64x64, 4 waves, 4-stage ring";
         case KERNEL_SPLIT_64x128: return "split-K 64x128x64, 4 waves, 4-stage ring";

@@ -142,8 +142,9 @@ __device__ __forceinline__ void store_wave_tile(const Acc (&acc)[Cfg::PTM][Cfg::
     constexpr int STRIP_ROW_BYTES = WN * 2 + 16;
     constexpr int STRIP_BYTES = 32 * STRIP_ROW_BYTES;  // sized for the 32-row case
     constexpr int LANES_PER_ROW = WN / 8;
-    constexpr int ROWS_PER_READ = 64 / LANES_PER_ROW;
-    constexpr int READS = MI / ROWS_PER_READ;
+    constexpr int ROWS_PER_READ = 64 / LANES_PER_ROW;                   // lanes beyond that many rows idle
+    constexpr int READS = (MI + ROWS_PER_READ - 1) / ROWS_PER_READ;
+    constexpr bool EXACT = (64 % LANES_PER_ROW == 0) && (MI % ROWS_PER_READ == 0);
     static_assert(STRIP_BYTES == Cfg::C_STRIP_BYTES, "strip size");
     unsigned char *strip = lds + wave * STRIP_BYTES;
     unsigned char *wr = strip + (lane % MI) * STRIP_ROW_BYTES + ((lane / MI) << 3);
@@ -163,16 +164,19 @@ __device__ __forceinline__ void store_wave_tile(const Acc (&acc)[Cfg::PTM][Cfg::
             }
 #pragma unroll
         for (int it = 0; it < READS; ++it) {
-            const u32x4 v = *reinterpret_cast<const u32x4 *>(rd + it * ROWS_PER_READ * STRIP_ROW_BYTES);
-            *reinterpret_cast<u32x4 *>(cp + (size_t)(i * MI + it * ROWS_PER_READ) * N) = v;
+            if (EXACT || (rd_row < ROWS_PER_READ && it * ROWS_PER_READ + rd_row < MI)) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(rd + it * ROWS_PER_READ * STRIP_ROW_BYTES);
+                *reinterpret_cast<u32x4 *>(cp + (size_t)(i * MI + it * ROWS_PER_READ) * N) = v;
+            }
         }
     }
 }
 
-template <class Cfg>
+template <class Cfg, bool SPLIT = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
-    hgemm_pipelined_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C, int M,
-                           int N, int K, int tiles_m, int tiles_n, long long *trace) {
+    hgemm_pipelined_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
+                           float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n,
+                           long long *trace) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
     constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS, CPR = Cfg::CPR, CPS = Cfg::CPS;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES, SA = Cfg::SA, SB = Cfg::SB;
@@ -181,7 +185,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     constexpr int NFRAG = TM + TN, NMMA = TM * TN;
     typedef typename MfmaOp<MI>::Acc Acc;
     static_assert(NFRAG <= NMMA, "at most one operand read is issued per MFMA slot");
-    (void)M;
+    static_assert(!SPLIT || MI == 16, "fp32 partial stores are written for the 16x16x32 accumulator layout");
     long long t_begin = 0, t_loop = 0, t_epi = 0, c_loop = 0, c_epi = 0;
     if (trace) t_begin = wall_clock64();
 
@@ -195,11 +199,12 @@ __global__ void __launch_bounds__(Cfg::THREADS)
 
     int tile_m, tile_n;
     tile_of_block<Cfg>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
-    const int num_k = K / BK;
+    const int num_k = k_len / BK;
+    const int k_begin = SPLIT ? (int)blockIdx.y * k_len : 0;
 
     // ---- copy set-up: wave w, instruction i fills LDS rows [(i*WAVES + w)*ROWS_PER_DMA, +ROWS_PER_DMA)
-    const unsigned char *a_base = reinterpret_cast<const unsigned char *>(A + (size_t)tile_m * BM * K);
-    const unsigned char *b_base = reinterpret_cast<const unsigned char *>(B + (size_t)tile_n * BN * K);
+    const unsigned char *a_base = reinterpret_cast<const unsigned char *>(A + (size_t)tile_m * BM * K + k_begin);
+    const unsigned char *b_base = reinterpret_cast<const unsigned char *>(B + (size_t)tile_n * BN * K + k_begin);
     constexpr int DMA_ROW_STEP = Cfg::WAVES * Cfg::ROWS_PER_DMA;
     uint32_t voff[L];
     {
@@ -287,6 +292,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             constexpr int t = decltype(g)::value * 4;
             lds_wait_all(a_frag[buf][t], a_frag[buf][t + 1], a_frag[buf][t + 2], a_frag[buf][t + 3]);
         });
+        static_for<TM % 4>([&](auto r) { lds_wait_all(a_frag[buf][TM / 4 * 4 + decltype(r)::value]); });
         static_for<NSB>([&](auto t) { lds_wait_all(b_frag[decltype(t)::value]); });
         static_for<NDB>([&](auto t) { lds_wait_all(b_last[buf][decltype(t)::value]); });
     };
@@ -455,8 +461,22 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         t_epi = wall_clock64();
         c_epi = clock64();
     }
-    __syncthreads();
-    store_wave_tile<Cfg, Acc>(acc, lds, C, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN, wave, lane);
+    if constexpr (SPLIT) {
+        // a lane holds four consecutive n of row m = lane % 16 of each 16x16 tile: 16 bytes of fp32
+        float *dst = partial + ((size_t)blockIdx.y * M + tile_m * BM + wm * Cfg::WM + lane % MI) * N + tile_n * BN +
+                     wn * Cfg::WN + (lane / MI) * 4;
+        static_for<TM>([&](auto i_c) {
+            static_for<TN>([&](auto j_c) {
+                constexpr int i = decltype(i_c)::value, j = decltype(j_c)::value;
+                *reinterpret_cast<floatx4 *>(dst + (size_t)(i * MI) * N + j * MI) = acc[i][j];
+            });
+        });
+    } else {
+        (void)M;
+        (void)partial;
+        __syncthreads();
+        store_wave_tile<Cfg, Acc>(acc, lds, C, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN, wave, lane);
+    }
     if (trace && tid == 0) {
         __builtin_amdgcn_s_waitcnt(0);
         long long *t = trace + (size_t)blockIdx.x * 8;
@@ -478,15 +498,40 @@ void launch_pipelined(const void *A, const void *B, void *C, size_t M, size_t N,
                     "%s needs M %% %d == 0, N %% %d == 0, K %% %d == 0, K >= %d (got M=%zu N=%zu K=%zu)", name,
                     Cfg::BM, Cfg::BN, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
     static bool configured = [] {
-        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg>),
+        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg, false>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
         return true;
     }();
     (void)configured;
     const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
-    hgemm_pipelined_kernel<Cfg><<<dim3(tiles_m * tiles_n), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
-        reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
-        (int)M, (int)N, (int)K, tiles_m, tiles_n, trace);
+    hgemm_pipelined_kernel<Cfg, false><<<dim3(tiles_m * tiles_n), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
+        reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), nullptr,
+        (int)M, (int)N, (int)K, (int)K, tiles_m, tiles_n, trace);
+    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+}
+
+// K split into `splits` slices: fp32 partial sums of slice s go to partial[s][M][N] (the
+// caller provides splits * M * N floats and runs the reduction afterwards).
+template <class Cfg>
+void launch_pipelined_split(const void *A, const void *B, float *partial, size_t M, size_t N, size_t K, int splits,
+                            const char *name) {
+    HGEMM_CHECK(splits >= 1 && K % (size_t)splits == 0);
+    const size_t k_len = K / (size_t)splits;
+    HGEMM_CHECK_MSG(Cfg::supports(M, N, k_len) && partial != nullptr,
+                    "%s (K in %d slices) needs M %% %d == 0, N %% %d == 0, slice %% %d == 0, slice >= %d "
+                    "(got M=%zu N=%zu K=%zu)",
+                    name, splits, Cfg::BM, Cfg::BN, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
+    static bool configured = [] {
+        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg, true>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        return true;
+    }();
+    (void)configured;
+    const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
+    hgemm_pipelined_kernel<Cfg, true>
+        <<<dim3(tiles_m * tiles_n, splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
+            reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), nullptr, partial, (int)M, (int)N,
+            (int)K, (int)k_len, tiles_m, tiles_n, nullptr);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 

@@ -17,6 +17,8 @@ enum KernelId {
     KERNEL_SPLIT_128x64,
     KERNEL_SPLIT_128x128,
     KERNEL_SIMT,        // scalar fallback for shapes no MFMA kernel tiles
+    KERNEL_T192,        // pipelined 192x192x64, 4 waves, 3-stage ring
+    KERNEL_R256x128,    // pipelined 256x128x64, 4 waves, 3-stage ring
 };
 
 struct Plan {

@@ -164,6 +164,27 @@ def test_auto_16384_sampled_rows(oracle, hgemm_lib, gpu):
     _sampled_check(oracle, got, A, B, n, rows_per_slab=8, slabs=2)
 
 
+@pytest.mark.parametrize("shape,tile,split", [
+    ((3072, 3072, 256), "192x192x64", False), ((2560, 2560, 256), "256x128x64", False),
+    ((256, 256, 8192), "64x64x64", True), ((1024, 1024, 4096), "128x128x64", True),
+    ((512, 512, 8192), "128x128x64", True), ((1536, 1536, 16384), "192x192x64", True),
+    ((2048, 2048, 16384), "256x256x64", True)])
+def test_auto_every_tile_with_and_without_k_slices(oracle, hgemm_lib, gpu, shape, tile, split):
+    """Shapes chosen so the dispatcher's cost model lands on each pipelined tile, alone and
+    with K cut into slices (fp32 partial sums + ordered reduction)."""
+    M, N, K = shape
+    plan = hgemm_lib.auto_plan(M, N, K)
+    assert tile in plan["kernel"] and (plan["splits"] > 1) == split, plan
+    A, B = oracle.fill((M, K), 21, 1), oracle.fill((N, K), 21, 2)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    _assert_close(oracle, first, oracle.hgemm(A, B), K)
+    assert np.array_equal(first, second)
+    At, Bt = oracle.fill((M, K), 22, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 22, 2, oracle.TERNARY, 0, 1)
+    ref = oracle.hgemm(At, Bt)
+    assert np.abs(ref.view(np.float16).astype(np.float32)).max() <= 2048      # integers exact in fp16
+    assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), ref)
+
+
 @pytest.mark.parametrize("N", [4096, 28672])
 @pytest.mark.parametrize("M", [1, 8, 16, 64, 128])
 def test_decode_shapes(oracle, hgemm_lib, gpu, M, N):
