@@ -52,13 +52,7 @@ void launch_splitk(const void *A, const void *B, void *C, size_t M, size_t N, si
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
         partial, (int)M, (int)N, (int)K, (int)(K / splits));
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
-    if (splits > 1) {
-        const size_t elems = M * N;
-        const unsigned blocks = (unsigned)div_ceil(elems / 8, 256);
-        splitk_reduce_kernel<<<dim3(blocks), dim3(256), 0, nullptr>>>(partial, reinterpret_cast<half_t *>(C), elems,
-                                                                      splits);
-        HGEMM_CHECK_HIP_ERROR(hipGetLastError());
-    }
+    if (splits > 1) launch_splitk_reduce(partial, reinterpret_cast<half_t *>(C), M * N, splits);
 }
 
 //                             BM   BN  WM WN stages
@@ -87,15 +81,12 @@ void launch_pipelined_plan(const void *A, const void *B, void *C, size_t M, size
     }
     float *partial = splitk_workspace((size_t)splits * M * N * sizeof(float));
     launch_pipelined_split<Cfg>(A, B, partial, M, N, K, splits, "hgemm_auto");
-    const size_t elems = M * N;  // a multiple of 8: every tile dimension is
-    splitk_reduce_kernel<<<dim3((unsigned)div_ceil(elems / 8, 256)), dim3(256), 0, nullptr>>>(
-        partial, reinterpret_cast<half_t *>(C), elems, splits);
-    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+    launch_splitk_reduce(partial, reinterpret_cast<half_t *>(C), M * N, splits);
 }
 
 // ---- cost model for the tile-aligned shapes.  A candidate is a tile (its kernel), how
 // many of its workgroups a CU holds, and three times in microseconds fitted to
-// measurements on an MI355X over ~60 shapes (rms error 7 %): `fix` per workgroup
+// measurements on an MI355X over ~50 shapes (rms error 6 %): `fix` per workgroup
 // (prologue, epilogue, scheduling) and the time of one 64-wide K chunk with few (`lo`)
 // and with all (`hi`) CUs busy -- the chip is power-limited, so a chunk costs more when
 // the whole chip computes.  time = launch + full rounds * (fix + chunks * hi)
@@ -106,13 +97,14 @@ struct Candidate {
     double fix, lo, hi;
 };
 constexpr Candidate CANDIDATES[] = {
-    {KERNEL_BIG256, 256, 256, 1, 2, 7.02, 0.959, 1.567},
-    {KERNEL_T192, 192, 192, 1, 3, 4.79, 0.585, 1.036},
-    {KERNEL_R256x128, 256, 128, 1, 3, 3.83, 0.561, 0.924},
-    {KERNEL_MID128, 128, 128, 1, 5, 2.99, 0.340, 0.543},
-    {KERNEL_SMALL64, 64, 64, 3, 3, 1.61, 0.394, 0.604},
+    {KERNEL_BIG256, 256, 256, 1, 2, 7.53, 0.978, 1.583},
+    {KERNEL_T192, 192, 192, 1, 3, 4.80, 0.605, 1.045},
+    {KERNEL_R256x128, 256, 128, 1, 3, 4.23, 0.579, 0.930},
+    {KERNEL_MID128, 128, 128, 1, 5, 3.29, 0.350, 0.551},
+    {KERNEL_SMALL64, 64, 64, 3, 3, 1.56, 0.398, 0.611},
 };
-constexpr double LAUNCH_US = 0.38, REDUCE_US = 4.86, REDUCE_BYTES_PER_US = 7207e3;
+// launch; reduction kernel: fixed + per slice + fp32 partials written and read back
+constexpr double LAUNCH_US = 0.11, REDUCE_US = 2.64, REDUCE_SLICE_US = 0.15, REDUCE_BYTES_PER_US = 7354e3;
 constexpr size_t MAX_PARTIAL_BYTES = 512ull << 20;
 
 double predict_us(const Candidate &c, size_t M, size_t N, size_t K, int splits, size_t cus) {
@@ -121,7 +113,8 @@ double predict_us(const Candidate &c, size_t M, size_t N, size_t K, int splits, 
     const size_t full = wgs / slots, rem = wgs % slots;
     double t = LAUNCH_US + (double)full * (c.fix + chunks * c.hi);
     if (rem) t += c.fix + chunks * (c.lo + (c.hi - c.lo) * (double)rem / (double)slots);
-    if (splits > 1) t += REDUCE_US + (double)splits * (double)M * (double)N * 8.0 / REDUCE_BYTES_PER_US;
+    if (splits > 1)
+        t += REDUCE_US + REDUCE_SLICE_US * splits + (double)splits * (double)M * (double)N * 8.0 / REDUCE_BYTES_PER_US;
     return t;
 }
 

@@ -150,24 +150,49 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     }
 }
 
-// C[i] = fp16( partial[0][i] + partial[1][i] + ... ) in slice order, 8 outputs per thread.
+// C[i] = fp16( partial[0][i] + partial[1][i] + ... ), always added in slice order, VEC
+// outputs per thread.  The loads of four slices are issued together before their adds, so
+// the kernel is not one memory round trip per slice; small outputs use a small VEC so the
+// reduction still spreads over the chip.
+template <int VEC>
 __global__ void __launch_bounds__(256)
     splitk_reduce_kernel(const float *__restrict__ partial, half_t *__restrict__ C, size_t elems, int splits) {
-    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
+    typedef half_t hvec_t __attribute__((ext_vector_type(VEC)));
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     if (i >= elems) return;
-    floatx4 s0 = *reinterpret_cast<const floatx4 *>(partial + i);
-    floatx4 s1 = *reinterpret_cast<const floatx4 *>(partial + i + 4);
-    for (int s = 1; s < splits; ++s) {
-        s0 += *reinterpret_cast<const floatx4 *>(partial + (size_t)s * elems + i);
-        s1 += *reinterpret_cast<const floatx4 *>(partial + (size_t)s * elems + i + 4);
+    const float *src = partial + i;
+    vec_t acc = *reinterpret_cast<const vec_t *>(src);
+    int s = 1;
+    for (; s + 4 <= splits; s += 4) {
+        const vec_t v0 = *reinterpret_cast<const vec_t *>(src + (size_t)s * elems);
+        const vec_t v1 = *reinterpret_cast<const vec_t *>(src + (size_t)(s + 1) * elems);
+        const vec_t v2 = *reinterpret_cast<const vec_t *>(src + (size_t)(s + 2) * elems);
+        const vec_t v3 = *reinterpret_cast<const vec_t *>(src + (size_t)(s + 3) * elems);
+        acc += v0;
+        acc += v1;
+        acc += v2;
+        acc += v3;
     }
-    half8 v;
+    for (; s < splits; ++s) acc += *reinterpret_cast<const vec_t *>(src + (size_t)s * elems);
+    hvec_t out;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        v[r] = (half_t)s0[r];
-        v[4 + r] = (half_t)s1[r];
-    }
-    *reinterpret_cast<half8 *>(C + i) = v;
+    for (int r = 0; r < VEC; ++r) out[r] = (half_t)acc[r];
+    *reinterpret_cast<hvec_t *>(C + i) = out;
+}
+
+// elems must be a multiple of 8 (every tile dimension is).
+inline void launch_splitk_reduce(const float *partial, half_t *C, size_t elems, int splits) {
+    if (elems >= (size_t)2 << 20)
+        splitk_reduce_kernel<8><<<dim3((unsigned)div_ceil(elems / 8, 256)), dim3(256), 0, nullptr>>>(partial, C, elems,
+                                                                                                    splits);
+    else if (elems >= (size_t)512 << 10)
+        splitk_reduce_kernel<4><<<dim3((unsigned)div_ceil(elems / 4, 256)), dim3(256), 0, nullptr>>>(partial, C, elems,
+                                                                                                    splits);
+    else
+        splitk_reduce_kernel<2><<<dim3((unsigned)div_ceil(elems / 2, 256)), dim3(256), 0, nullptr>>>(partial, C, elems,
+                                                                                                    splits);
+    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 
 }  // namespace hgemm
