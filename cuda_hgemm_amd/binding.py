@@ -67,6 +67,8 @@ def _tensor_ptr(t, rows: int, cols: int, what: str) -> int:
         raise ValueError(f"{what}: expected shape {(rows, cols)}, got {tuple(t.shape)}")
     if not t.is_contiguous():
         raise ValueError(f"{what}: must be contiguous")
+    if t.data_ptr() % 16:
+        raise ValueError(f"{what}: must start on a 16-byte boundary")
     return t.data_ptr()
 
 

@@ -91,6 +91,9 @@ inline void check_operands(const void *A, const void *B, const void *C, size_t M
     HGEMM_CHECK_GT(M, 0u);
     HGEMM_CHECK_GT(N, 0u);
     HGEMM_CHECK_GT(K, 0u);
+    // 16-byte vector accesses start at the operand bases (hipMalloc returns 256-byte alignment).
+    HGEMM_CHECK_MSG((((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) == 0,
+                    "A, B and C must be 16-byte aligned (got %p %p %p)", A, B, C);
     // Kernels index with 32-bit element offsets inside one operand.
     HGEMM_CHECK_MSG(M * K < (1ull << 31) && N * K < (1ull << 31) && M * N < (1ull << 31),
                     "operand with more than 2^31 elements (M=%zu N=%zu K=%zu)", M, N, K);

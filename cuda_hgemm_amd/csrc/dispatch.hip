@@ -1,6 +1,7 @@
 // hgemm_skinny and hgemm_auto: shape-driven choice among the tuned kernels.
 #include "../../include/hgemm.h"
 #include "mfma_pipelined.h"
+#include "mfma_ragged.h"
 #include "mfma_skinny.h"
 #include "plan.h"
 
@@ -108,7 +109,8 @@ constexpr double LAUNCH_US = 0.11, REDUCE_US = 2.64, REDUCE_SLICE_US = 0.15, RED
 constexpr size_t MAX_PARTIAL_BYTES = 512ull << 20;
 
 double predict_us(const Candidate &c, size_t M, size_t N, size_t K, int splits, size_t cus) {
-    const size_t wgs = (M / c.bm) * (N / c.bn) * (size_t)splits, slots = cus * (size_t)c.per_cu;
+    const size_t wgs = div_ceil(M, (size_t)c.bm) * div_ceil(N, (size_t)c.bn) * (size_t)splits;
+    const size_t slots = cus * (size_t)c.per_cu;
     const double chunks = (double)(K / (size_t)splits / 64);
     const size_t full = wgs / slots, rem = wgs % slots;
     double t = LAUNCH_US + (double)full * (c.fix + chunks * c.hi);
@@ -156,9 +158,11 @@ Plan plan_for(size_t M, size_t N, size_t K) {
         p.splits = choose_splits(N / (wide ? 128 : 64), cus, K);
         return p;
     }
+    // Pipelined tiles: M and N may end inside a tile (guarded edges; the model charges whole
+    // tiles), as long as rows of C stay 16-byte aligned and K is a whole number of chunks.
     double best = 0.0;
     for (const Candidate &c : CANDIDATES) {
-        if (M % c.bm || N % c.bn) continue;
+        if (N % 8) break;
         for (int s = 1; s <= 32; s *= 2) {
             if (K % ((size_t)s * 64) || K / s < (size_t)64 * c.stages) break;
             if (s > 1 && (size_t)s * M * N * sizeof(float) > MAX_PARTIAL_BYTES) break;
@@ -176,7 +180,7 @@ Plan plan_for(size_t M, size_t N, size_t K) {
         p.splits = choose_splits(div_ceil(M, 64) * (N / 64), cus, K);
         return p;
     }
-    p.kernel = KERNEL_SIMT;
+    p.kernel = KERNEL_RAGGED;
     return p;
 }
 
@@ -193,6 +197,7 @@ void run_plan(const Plan &p, const void *A, const void *B, void *C, size_t M, si
         case KERNEL_SPLIT_64x128: launch_splitk<Split64x128>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_SPLIT_128x64: launch_splitk<Split128x64>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_SPLIT_128x128: launch_splitk<Split128x128>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_RAGGED: launch_ragged(A, B, C, M, N, K); break;
         case KERNEL_SIMT:
             hgemm_simt_naive(reinterpret_cast<const hgemm_half *>(A), reinterpret_cast<const hgemm_half *>(B),
                              reinterpret_cast<hgemm_half *>(C), M, N, K);
@@ -238,6 +243,7 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
         case KERNEL_SPLIT_64x128: return "split-K 64x128x64, 4 waves, 4-stage ring";
         case KERNEL_SPLIT_128x64: return "split-K 128x64x64, 4 waves, 4-stage ring";
         case KERNEL_SPLIT_128x128: return "split-K 128x128x64, 4 waves, 4-stage ring";
+        case KERNEL_RAGGED: return "guarded 128x128x32, 4 waves, any shape";
         case KERNEL_SIMT: return "scalar fallback";
         default: return "none";
     }

@@ -133,9 +133,10 @@ __device__ __forceinline__ void dma_load16_sv(const void *sbase, uint32_t voff, 
 // holds groups of four consecutive n of one row m = lane % MI): each wave parks MI rows of
 // its tile in a private strip and reads them back row-contiguous, 16 bytes per lane, so a
 // global store instruction writes whole 128-byte lines.
-template <class Cfg, class Acc>
+// EDGE: rows >= M and 8-column pieces at or beyond N (N % 8 == 0) are not stored.
+template <class Cfg, class Acc, bool EDGE = false>
 __device__ __forceinline__ void store_wave_tile(const Acc (&acc)[Cfg::PTM][Cfg::PTN], unsigned char *lds,
-                                                half_t *__restrict__ C, int N, int row0, int col0, int wave,
+                                                half_t *__restrict__ C, int M, int N, int row0, int col0, int wave,
                                                 int lane) {
     constexpr int MI = Cfg::MI, TM = Cfg::PTM, TN = Cfg::PTN, WN = Cfg::WN;
     constexpr int GROUPS = MI == 32 ? 4 : 1;          // register groups of four n per accumulator
@@ -166,13 +167,17 @@ __device__ __forceinline__ void store_wave_tile(const Acc (&acc)[Cfg::PTM][Cfg::
         for (int it = 0; it < READS; ++it) {
             if (EXACT || (rd_row < ROWS_PER_READ && it * ROWS_PER_READ + rd_row < MI)) {
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(rd + it * ROWS_PER_READ * STRIP_ROW_BYTES);
-                *reinterpret_cast<u32x4 *>(cp + (size_t)(i * MI + it * ROWS_PER_READ) * N) = v;
+                if (!EDGE || (row0 + rd_row + i * MI + it * ROWS_PER_READ < M && col0 + rd_col * 8 < N))
+                    *reinterpret_cast<u32x4 *>(cp + (size_t)(i * MI + it * ROWS_PER_READ) * N) = v;
             }
         }
     }
 }
 
-template <class Cfg, bool SPLIT = false>
+// EDGE: M and N need not be multiples of the tile (N % 8 == 0 still, for aligned rows of
+// C).  Copies of rows beyond the matrix are redirected to its last row -- valid memory,
+// products never stored -- which costs nothing inside the loop; only the stores are guarded.
+template <class Cfg, bool SPLIT = false, bool EDGE = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_pipelined_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
                            float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n,
@@ -211,17 +216,20 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         // lane l of instruction `it` lands on physical chunk l % CPR of LDS row
         // row0 + it * DMA_ROW_STEP, so it fetches the logical chunk the swizzle maps there
         const int row0 = wave * Cfg::ROWS_PER_DMA + lane / CPR;
+        const int last_a = M - 1 - tile_m * BM, last_b = N - 1 - tile_n * BN;  // last valid row of the tile
 #pragma unroll
         for (int it = 0; it < A_DMA; ++it) {
             const int row = row0 + it * DMA_ROW_STEP;
             const int ch = (lane % CPR) ^ swizzle_of_row<Cfg>(row);
-            voff[it] = ((uint32_t)row * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
+            const int src = (EDGE && row > last_a) ? last_a : row;
+            voff[it] = ((uint32_t)src * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
         }
 #pragma unroll
         for (int it = 0; it < B_DMA; ++it) {
             const int row = row0 + it * DMA_ROW_STEP;
             const int ch = (lane % CPR) ^ swizzle_of_row<Cfg>(row);
-            voff[A_DMA + it] = ((uint32_t)row * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
+            const int src = (EDGE && row > last_b) ? last_b : row;
+            voff[A_DMA + it] = ((uint32_t)src * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
         }
     }
     const uint32_t cp_lds = lds_base + wave * 1024;
@@ -463,19 +471,20 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     }
     if constexpr (SPLIT) {
         // a lane holds four consecutive n of row m = lane % 16 of each 16x16 tile: 16 bytes of fp32
-        float *dst = partial + ((size_t)blockIdx.y * M + tile_m * BM + wm * Cfg::WM + lane % MI) * N + tile_n * BN +
-                     wn * Cfg::WN + (lane / MI) * 4;
+        const int row = tile_m * BM + wm * Cfg::WM + lane % MI, col = tile_n * BN + wn * Cfg::WN + (lane / MI) * 4;
+        float *dst = partial + ((size_t)blockIdx.y * M + row) * N + col;
         static_for<TM>([&](auto i_c) {
             static_for<TN>([&](auto j_c) {
                 constexpr int i = decltype(i_c)::value, j = decltype(j_c)::value;
-                *reinterpret_cast<floatx4 *>(dst + (size_t)(i * MI) * N + j * MI) = acc[i][j];
+                if (!EDGE || (row + i * MI < M && col + j * MI < N))
+                    *reinterpret_cast<floatx4 *>(dst + (size_t)(i * MI) * N + j * MI) = acc[i][j];
             });
         });
     } else {
-        (void)M;
         (void)partial;
         __syncthreads();
-        store_wave_tile<Cfg, Acc>(acc, lds, C, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN, wave, lane);
+        store_wave_tile<Cfg, Acc, EDGE>(acc, lds, C, M, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN,
+                                        wave, lane);
     }
     if (trace && tid == 0) {
         __builtin_amdgcn_s_waitcnt(0);
@@ -490,24 +499,43 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     }
 }
 
+// Shapes a pipelined kernel accepts with guarded edges: any M, N a multiple of 8 (rows of C
+// stay 16-byte aligned), K a whole number of chunks and at least the ring depth.
+template <class Cfg>
+bool pipelined_supports_edges(size_t M, size_t N, size_t K) {
+    return M > 0 && N > 0 && N % 8 == 0 && K % Cfg::BK == 0 && K >= (size_t)Cfg::BK * Cfg::STAGES;
+}
+
+template <class Cfg, bool SPLIT, bool EDGE>
+void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial, size_t M, size_t N, size_t K,
+                           int splits, long long *trace) {
+    static bool configured = [] {
+        HGEMM_CHECK_HIP_ERROR(
+            hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg, SPLIT, EDGE>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        return true;
+    }();
+    (void)configured;
+    const int tiles_m = (int)div_ceil(M, (size_t)Cfg::BM), tiles_n = (int)div_ceil(N, (size_t)Cfg::BN);
+    hgemm_pipelined_kernel<Cfg, SPLIT, EDGE>
+        <<<dim3(tiles_m * tiles_n, splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
+            reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
+            partial, (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, trace);
+    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+}
+
 template <class Cfg>
 void launch_pipelined(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, const char *name,
                       long long *trace = nullptr) {
     check_operands(A, B, C, M, N, K);
-    HGEMM_CHECK_MSG(Cfg::supports(M, N, K),
-                    "%s needs M %% %d == 0, N %% %d == 0, K %% %d == 0, K >= %d (got M=%zu N=%zu K=%zu)", name,
-                    Cfg::BM, Cfg::BN, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
-    static bool configured = [] {
-        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg, false>),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
-        return true;
-    }();
-    (void)configured;
-    const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
-    hgemm_pipelined_kernel<Cfg, false><<<dim3(tiles_m * tiles_n), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
-        reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), nullptr,
-        (int)M, (int)N, (int)K, (int)K, tiles_m, tiles_n, trace);
-    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+    if (Cfg::supports(M, N, K)) {
+        launch_pipelined_impl<Cfg, false, false>(A, B, C, nullptr, M, N, K, 1, trace);
+        return;
+    }
+    HGEMM_CHECK_MSG(pipelined_supports_edges<Cfg>(M, N, K),
+                    "%s needs N %% 8 == 0, K %% %d == 0, K >= %d (got M=%zu N=%zu K=%zu)", name, Cfg::BK,
+                    Cfg::BK * Cfg::STAGES, M, N, K);
+    launch_pipelined_impl<Cfg, false, true>(A, B, C, nullptr, M, N, K, 1, trace);
 }
 
 // K split into `splits` slices: fp32 partial sums of slice s go to partial[s][M][N] (the
@@ -515,24 +543,16 @@ void launch_pipelined(const void *A, const void *B, void *C, size_t M, size_t N,
 template <class Cfg>
 void launch_pipelined_split(const void *A, const void *B, float *partial, size_t M, size_t N, size_t K, int splits,
                             const char *name) {
-    HGEMM_CHECK(splits >= 1 && K % (size_t)splits == 0);
+    HGEMM_CHECK(splits >= 1 && K % (size_t)splits == 0 && partial != nullptr);
     const size_t k_len = K / (size_t)splits;
-    HGEMM_CHECK_MSG(Cfg::supports(M, N, k_len) && partial != nullptr,
-                    "%s (K in %d slices) needs M %% %d == 0, N %% %d == 0, slice %% %d == 0, slice >= %d "
-                    "(got M=%zu N=%zu K=%zu)",
-                    name, splits, Cfg::BM, Cfg::BN, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
-    static bool configured = [] {
-        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg, true>),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
-        return true;
-    }();
-    (void)configured;
-    const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
-    hgemm_pipelined_kernel<Cfg, true>
-        <<<dim3(tiles_m * tiles_n, splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
-            reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), nullptr, partial, (int)M, (int)N,
-            (int)K, (int)k_len, tiles_m, tiles_n, nullptr);
-    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+    if (Cfg::supports(M, N, k_len)) {
+        launch_pipelined_impl<Cfg, true, false>(A, B, nullptr, partial, M, N, K, splits, nullptr);
+        return;
+    }
+    HGEMM_CHECK_MSG(pipelined_supports_edges<Cfg>(M, N, k_len),
+                    "%s (K in %d slices) needs N %% 8 == 0, slice %% %d == 0, slice >= %d (got M=%zu N=%zu K=%zu)",
+                    name, splits, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
+    launch_pipelined_impl<Cfg, true, true>(A, B, nullptr, partial, M, N, K, splits, nullptr);
 }
 
 }  // namespace hgemm

@@ -19,6 +19,7 @@ enum KernelId {
     KERNEL_SIMT,        // scalar fallback for shapes no MFMA kernel tiles
     KERNEL_T192,        // pipelined 192x192x64, 4 waves, 3-stage ring
     KERNEL_R256x128,    // pipelined 256x128x64, 4 waves, 3-stage ring
+    KERNEL_RAGGED,      // guarded 128x128x32 MFMA kernel: any shape
 };
 
 struct Plan {

@@ -11,7 +11,8 @@
  *     A  row-major   M x K                      (reference src/common/tester.h:117)
  *     B  column-major K x N, i.e. N rows of K    (reference src/common/tester.h:118)
  *     C  row-major   M x N, fully overwritten    (reference src/common/tester.h:119)
- * Elements are IEEE binary16 (2 bytes).  Products are accumulated in fp32 and rounded to
+ * Elements are IEEE binary16 (2 bytes); A, B and C start on 16-byte boundaries (hipMalloc
+ * gives 256).  Products are accumulated in fp32 and rounded to
  * fp16 once (the reference accumulates in fp16; this is the one deliberate difference).
  *
  * Calling convention, as in the reference (src/mma/mma_async_stage4.cu:637-644,
@@ -84,9 +85,10 @@ HGEMM_FUNC(hgemm_mfma_async_stage4);
  * (reference src/mma/mma_async_stage4.cu:64-66,93-94). */
 HGEMM_FUNC(hgemm_skinny);
 
-/* Dispatcher: picks the tile / kernel for the shape; accepts every shape with
- * K % 8 == 0 through the MFMA kernels and anything else through the scalar kernel.
- * This is the entry point the benchmark measures. */
+/* Dispatcher: picks tile, kernel and number of K slices for the shape from a cost model
+ * fitted to measurements; accepts every shape.  N % 8 == 0 and K % 64 == 0 run on the
+ * pipelined kernels (M and N may end inside a tile: edges are guarded), anything else on a
+ * fully guarded MFMA kernel.  This is the entry point the benchmark measures. */
 HGEMM_FUNC(hgemm_auto);
 
 /* Kernel hgemm_auto would pick for a shape (an id for hgemm_kernel_name) and, through

@@ -208,11 +208,40 @@ def test_skinny_ragged_M(oracle, hgemm_lib, gpu, M):
     assert np.array_equal(_run(hgemm_lib, "hgemm_skinny", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
-@pytest.mark.parametrize("shape", [(100, 100, 100), (1, 7, 5), (257, 129, 33), (640, 384, 192), (192, 320, 4096)])
+RAGGED = [(100, 100, 100), (1, 7, 5), (3, 17, 33), (257, 129, 33), (640, 384, 192), (192, 320, 4096),
+          (300, 304, 64), (130, 250, 1000), (1000, 1000, 1000), (129, 4096, 512), (1000, 4000, 1024),
+          (1030, 520, 2048), (70, 72, 8192), (2100, 2056, 384), (515, 1032, 4100), (260, 1288, 6144)]
+
+
+@pytest.mark.parametrize("shape", RAGGED)
 def test_auto_handles_shapes_no_tile_divides(oracle, hgemm_lib, gpu, shape):
+    """M, N, K that end inside a tile: the pipelined kernels with guarded edges (N % 8 == 0,
+    K % 64 == 0, with and without K slices) and the fully guarded kernel for the rest.
+    Poisoned C shows any element left unwritten; exact ternary inputs show any element
+    taken from a wrong row or from beyond K."""
     M, N, K = shape
     A, B = oracle.fill((M, K), 13, 1), oracle.fill((N, K), 13, 2)
-    _assert_close(oracle, _run(hgemm_lib, "hgemm_auto", A, B, gpu), oracle.hgemm(A, B), K)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    _assert_close(oracle, first, oracle.hgemm(A, B), K)
+    assert np.array_equal(first, second)
+    At, Bt = oracle.fill((M, K), 14, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 14, 2, oracle.TERNARY, 0, 1)
+    assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
+
+
+def test_guarded_edges_do_not_write_outside_c(oracle, hgemm_lib, gpu):
+    """C sits inside a larger poisoned allocation: nothing before or after it may change."""
+    import torch
+    for (M, N, K) in [(1000, 1000, 1000), (1000, 4000, 1024), (130, 136, 8192)]:
+        A, B = oracle.fill((M, K), 15, 1), oracle.fill((N, K), 15, 2)
+        pad = 4096   # elements; keeps C 16-byte aligned
+        buf = torch.full((pad + M * N + pad,), POISON - 65536, dtype=torch.int16, device=gpu)
+        C = buf[pad:pad + M * N].view(torch.float16).view(M, N)
+        print(f"[gpu] hgemm_auto M={M} N={N} K={K} inside a guard band", flush=True)
+        hgemm_lib.call("hgemm_auto", _to_gpu(A, gpu), _to_gpu(B, gpu), C, M, N, K)
+        torch.cuda.synchronize()
+        host = buf.cpu().numpy().view(np.uint16)
+        assert np.all(host[:pad] == POISON) and np.all(host[pad + M * N:] == POISON)
+        _assert_close(oracle, host[pad:pad + M * N].reshape(M, N), oracle.hgemm(A, B), K)
 
 
 # ------------------------------------------------------------------ size-independent properties at full size
