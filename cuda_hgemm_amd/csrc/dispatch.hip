@@ -26,6 +26,21 @@ float *splitk_workspace(size_t bytes) {
     return ptr;
 }
 
+// Same, for zero-padded copies of the operands of shapes whose rows are not aligned.
+unsigned char *operand_workspace(size_t bytes) {
+    static unsigned char *ptr = nullptr;
+    static size_t capacity = 0;
+    if (bytes > capacity) {
+        if (ptr) {
+            HGEMM_CHECK_HIP_ERROR(hipDeviceSynchronize());
+            HGEMM_CHECK_HIP_ERROR(hipFree(ptr));
+        }
+        HGEMM_CHECK_HIP_ERROR(hipMalloc(reinterpret_cast<void **>(&ptr), bytes));
+        capacity = bytes;
+    }
+    return ptr;
+}
+
 int compute_units() {
     static int cus = [] {
         // A planning query must also work where no GPU is visible: assume one MI355X.
@@ -107,6 +122,14 @@ constexpr Candidate CANDIDATES[] = {
 // launch; reduction kernel: fixed + per slice + fp32 partials written and read back
 constexpr double LAUNCH_US = 0.11, REDUCE_US = 2.64, REDUCE_SLICE_US = 0.15, REDUCE_BYTES_PER_US = 7354e3;
 constexpr size_t MAX_PARTIAL_BYTES = 512ull << 20;
+constexpr size_t MAX_PADDED_BYTES = 1024ull << 20;
+size_t padded_n(size_t N) { return (N + 7) / 8 * 8; }
+size_t padded_k(size_t K) { return (K + 63) / 64 * 64; }
+// A' (M x K'), B' (N' x K') and, when N grows, C' (M x N')
+size_t padded_bytes(size_t M, size_t N, size_t K) {
+    const size_t Np = padded_n(N), Kp = padded_k(K);
+    return ((M + Np) * Kp + (Np != N ? M * Np : 0)) * sizeof(half_t);
+}
 
 double predict_us(const Candidate &c, size_t M, size_t N, size_t K, int splits, size_t cus) {
     const size_t wgs = div_ceil(M, (size_t)c.bm) * div_ceil(N, (size_t)c.bn) * (size_t)splits;
@@ -171,6 +194,7 @@ Plan plan_for(size_t M, size_t N, size_t K) {
                 best = t;
                 p.kernel = c.kernel;
                 p.splits = s;
+                p.est_us = t;
             }
         }
     }
@@ -180,8 +204,79 @@ Plan plan_for(size_t M, size_t N, size_t K) {
         p.splits = choose_splits(div_ceil(M, 64) * (N / 64), cus, K);
         return p;
     }
+    // Rows of C not 16-byte aligned (N % 8) or K not a whole number of chunks.  Large
+    // products are worth two extra passes over the operands: copy A and B zero-padded to a
+    // shape the pipelined kernels take and run that (same products, same result); the rest
+    // goes to the guarded kernel, which sustains about 80 TFLOP/s.
+    const size_t Np = padded_n(N), Kp = padded_k(K);
+    if (K >= 192 && padded_bytes(M, N, K) <= MAX_PADDED_BYTES) {
+        const Plan inner = plan_for(M, Np, Kp);
+        const double inner_us = inner.est_us > 0.0 ? inner.est_us : 8.0 + (double)(Np * Kp * 2) / 4e6;
+        const double copy_us = 6.0 + 4.0 * (double)((M + Np) * Kp + (Np != N ? M * Np : 0)) / 3.5e6;
+        const double guarded_us = 5.0 + 2.0 * (double)M * (double)N * (double)K / 80e6;
+        if (inner.kernel != KERNEL_RAGGED && inner.kernel != KERNEL_PADDED && copy_us + inner_us < guarded_us) {
+            p.kernel = KERNEL_PADDED;
+            p.splits = inner.splits;
+            p.est_us = copy_us + inner_us;
+            return p;
+        }
+    }
     p.kernel = KERNEL_RAGGED;
     return p;
+}
+
+// dst[r][0..cols_dst) = src[r][0..cols_src) followed by zeros, for r < rows_src; rows
+// beyond rows_src are all zeros.  One thread per 8 halves of dst.
+__global__ void __launch_bounds__(256)
+    pad_copy_kernel(const half_t *__restrict__ src, half_t *__restrict__ dst, int rows_src, int cols_src, int rows_dst,
+                    int cols_dst) {
+    const size_t chunk = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int chunks_per_row = cols_dst / 8;
+    const size_t row = chunk / chunks_per_row;
+    if (row >= (size_t)rows_dst) return;
+    const int col = (int)(chunk % chunks_per_row) * 8;
+    half8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (half_t)0.0f;
+    if (row < (size_t)rows_src && col < cols_src) {
+        const half_t *s = src + row * cols_src + col;
+        if ((cols_src & 7) == 0) {
+            v = *reinterpret_cast<const half8 *>(s);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (col + e < cols_src) v[e] = s[e];
+        }
+    }
+    *reinterpret_cast<half8 *>(dst + row * cols_dst + col) = v;
+}
+// dst[r][c] = src[r][c] for c < cols_dst <= cols_src (drops the padding columns of C).
+__global__ void __launch_bounds__(256)
+    unpad_copy_kernel(const half_t *__restrict__ src, half_t *__restrict__ dst, int rows, int cols_src, int cols_dst) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * cols_dst) return;
+    const size_t r = i / cols_dst, c = i % cols_dst;
+    dst[i] = src[r * cols_src + c];
+}
+
+void run_padded(const void *A, const void *B, void *C, size_t M, size_t N, size_t K) {
+    const size_t Np = padded_n(N), Kp = padded_k(K);
+    unsigned char *ws = operand_workspace(padded_bytes(M, N, K));
+    half_t *Ap = reinterpret_cast<half_t *>(ws), *Bp = Ap + M * Kp;
+    half_t *Cp = Np != N ? Bp + Np * Kp : reinterpret_cast<half_t *>(C);
+    pad_copy_kernel<<<dim3((unsigned)div_ceil(M * (Kp / 8), (size_t)256)), dim3(256), 0, nullptr>>>(
+        reinterpret_cast<const half_t *>(A), Ap, (int)M, (int)K, (int)M, (int)Kp);
+    pad_copy_kernel<<<dim3((unsigned)div_ceil(Np * (Kp / 8), (size_t)256)), dim3(256), 0, nullptr>>>(
+        reinterpret_cast<const half_t *>(B), Bp, (int)N, (int)K, (int)Np, (int)Kp);
+    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+    const Plan inner = plan_for(M, Np, Kp);
+    HGEMM_CHECK(inner.kernel != KERNEL_PADDED && inner.kernel != KERNEL_RAGGED);
+    run_plan(inner, Ap, Bp, Cp, M, Np, Kp);
+    if (Np != N) {
+        unpad_copy_kernel<<<dim3((unsigned)div_ceil(M * N, (size_t)256)), dim3(256), 0, nullptr>>>(
+            Cp, reinterpret_cast<half_t *>(C), (int)M, (int)Np, (int)N);
+        HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+    }
 }
 
 void run_plan(const Plan &p, const void *A, const void *B, void *C, size_t M, size_t N, size_t K) {
@@ -198,6 +293,7 @@ void run_plan(const Plan &p, const void *A, const void *B, void *C, size_t M, si
         case KERNEL_SPLIT_128x64: launch_splitk<Split128x64>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_SPLIT_128x128: launch_splitk<Split128x128>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_RAGGED: launch_ragged(A, B, C, M, N, K); break;
+        case KERNEL_PADDED: run_padded(A, B, C, M, N, K); break;
         case KERNEL_SIMT:
             hgemm_simt_naive(reinterpret_cast<const hgemm_half *>(A), reinterpret_cast<const hgemm_half *>(B),
                              reinterpret_cast<hgemm_half *>(C), M, N, K);
@@ -244,6 +340,7 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
         case KERNEL_SPLIT_128x64: return "split-K 128x64x64, 4 waves, 4-stage ring";
         case KERNEL_SPLIT_128x128: return "split-K 128x128x64, 4 waves, 4-stage ring";
         case KERNEL_RAGGED: return "guarded 128x128x32, 4 waves, any shape";
+        case KERNEL_PADDED: return "zero-padded operand copies + pipelined kernel of the padded shape";
         case KERNEL_SIMT: return "scalar fallback";
         default: return "none";
     }

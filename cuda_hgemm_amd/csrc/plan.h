@@ -20,11 +20,13 @@ enum KernelId {
     KERNEL_T192,        // pipelined 192x192x64, 4 waves, 3-stage ring
     KERNEL_R256x128,    // pipelined 256x128x64, 4 waves, 3-stage ring
     KERNEL_RAGGED,      // guarded 128x128x32 MFMA kernel: any shape
+    KERNEL_PADDED,      // operands copied zero-padded to N % 8 == 0, K % 64 == 0, then the plan for that shape
 };
 
 struct Plan {
     int kernel = KERNEL_NONE;
     int splits = 1;
+    double est_us = 0.0;  // the cost model's estimate where it was used, else 0
 };
 
 bool skinny_supports(size_t M, size_t N, size_t K);

@@ -89,6 +89,7 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
             assert 4096 % (p["splits"] * 64) == 0
     assert plan(100, 100, 100)["kernel"].startswith("guarded 128x128x32")      # no tile divides it
     assert plan(1000, 4000, 4096)["kernel"].startswith("pipelined")            # ragged M, N: guarded edges
+    assert plan(4095, 4095, 4095)["kernel"].startswith("zero-padded")          # large and unaligned
 
 
 def test_metrics(hgemm_lib):

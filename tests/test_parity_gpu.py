@@ -210,13 +210,15 @@ def test_skinny_ragged_M(oracle, hgemm_lib, gpu, M):
 
 RAGGED = [(100, 100, 100), (1, 7, 5), (3, 17, 33), (257, 129, 33), (640, 384, 192), (192, 320, 4096),
           (300, 304, 64), (130, 250, 1000), (1000, 1000, 1000), (129, 4096, 512), (1000, 4000, 1024),
-          (1030, 520, 2048), (70, 72, 8192), (2100, 2056, 384), (515, 1032, 4100), (260, 1288, 6144)]
+          (1030, 520, 2048), (70, 72, 8192), (2100, 2056, 384), (515, 1032, 4100), (260, 1288, 6144),
+          (2047, 2049, 2051), (2050, 2050, 2048), (64, 1023, 1022)]
 
 
 @pytest.mark.parametrize("shape", RAGGED)
 def test_auto_handles_shapes_no_tile_divides(oracle, hgemm_lib, gpu, shape):
     """M, N, K that end inside a tile: the pipelined kernels with guarded edges (N % 8 == 0,
-    K % 64 == 0, with and without K slices) and the fully guarded kernel for the rest.
+    K % 64 == 0, with and without K slices), zero-padded operand copies for large unaligned
+    shapes, and the fully guarded kernel for the rest.
     Poisoned C shows any element left unwritten; exact ternary inputs show any element
     taken from a wrong row or from beyond K."""
     M, N, K = shape
@@ -231,7 +233,7 @@ def test_auto_handles_shapes_no_tile_divides(oracle, hgemm_lib, gpu, shape):
 def test_guarded_edges_do_not_write_outside_c(oracle, hgemm_lib, gpu):
     """C sits inside a larger poisoned allocation: nothing before or after it may change."""
     import torch
-    for (M, N, K) in [(1000, 1000, 1000), (1000, 4000, 1024), (130, 136, 8192)]:
+    for (M, N, K) in [(1000, 1000, 1000), (1000, 4000, 1024), (130, 136, 8192), (100, 100, 100), (1026, 1030, 1100)]:
         A, B = oracle.fill((M, K), 15, 1), oracle.fill((N, K), 15, 2)
         pad = 4096   # elements; keeps C 16-byte aligned
         buf = torch.full((pad + M * N + pad,), POISON - 65536, dtype=torch.int16, device=gpu)
