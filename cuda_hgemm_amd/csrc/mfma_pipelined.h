@@ -57,6 +57,24 @@ struct PipeConfig : TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_
     }
 };
 
+// XOR applied to the 16-byte chunk index of LDS row `row`.  A ds_read_b128 serves its 64
+// lanes in four cycles of 16 lanes over 64 banks, and (measured with the LDS bank-conflict
+// counter) the 16 lanes of one cycle are lanes [8g, 8g+8) together with [32+8g, 32+8g+8).
+// With 16x16x32 operands (lane l reads row l % 16, chunk l / 16 of the step) and 128-byte
+// rows, one cycle therefore touches 8 rows at chunk c and the same 8 rows at chunk c ^ 2:
+// the four rows of equal parity must get XOR values from four different cosets of {0, 2},
+// which the row-number swizzle of the other kernels does not give (half of all LDS cycles
+// were conflicts).  Rows 8-15 use the complementary values, so 16 consecutive rows at one
+// chunk are conflict-free as well.
+template <class Cfg>
+__device__ __forceinline__ int pipe_swizzle(int row) {
+    if constexpr (Cfg::MI == 16 && Cfg::BK == 64) {
+        const int x = (row >> 1) & 3;
+        return ((x & 1) | ((x & 2) << 1)) ^ (((row >> 3) & 1) << 1);
+    }
+    return swizzle_of_row<Cfg>(row);
+}
+
 // Compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>).  The
 // pipeline body is laid out slot by slot with every index a constant; this does not lean
 // on the loop unroller, whose failure would turn the accumulators into scratch memory.
@@ -220,14 +238,14 @@ __global__ void __launch_bounds__(Cfg::THREADS)
 #pragma unroll
         for (int it = 0; it < A_DMA; ++it) {
             const int row = row0 + it * DMA_ROW_STEP;
-            const int ch = (lane % CPR) ^ swizzle_of_row<Cfg>(row);
+            const int ch = (lane % CPR) ^ pipe_swizzle<Cfg>(row);
             const int src = (EDGE && row > last_a) ? last_a : row;
             voff[it] = ((uint32_t)src * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
         }
 #pragma unroll
         for (int it = 0; it < B_DMA; ++it) {
             const int row = row0 + it * DMA_ROW_STEP;
-            const int ch = (lane % CPR) ^ swizzle_of_row<Cfg>(row);
+            const int ch = (lane % CPR) ^ pipe_swizzle<Cfg>(row);
             const int src = (EDGE && row > last_b) ? last_b : row;
             voff[A_DMA + it] = ((uint32_t)src * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
         }
@@ -249,7 +267,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     // ---- operand fragment set-up: lane l supplies 8 consecutive k (chunk l / MI of the
     // step) of row l % MI, for both operands.
     const int frag_row = lane % MI;
-    const int frag_x = (lane / MI) ^ swizzle_of_row<Cfg>(frag_row);
+    const int frag_x = (lane / MI) ^ pipe_swizzle<Cfg>(frag_row);
     const uint32_t a_frag_off = (wm * Cfg::WM + frag_row) * ROW_BYTES;
     const uint32_t b_frag_off = B_REGION + (wn * Cfg::WN + frag_row) * ROW_BYTES;
     // Fragment idx sits idx * MI rows further down.  That never changes bits 0-2 of the
