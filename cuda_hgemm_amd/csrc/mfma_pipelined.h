@@ -75,6 +75,13 @@ __device__ __forceinline__ int pipe_swizzle(int row) {
     return swizzle_of_row<Cfg>(row);
 }
 
+template <class T, T V>
+constexpr int ring_index(std::integral_constant<T, V>) {
+    return (int)V;
+}
+constexpr int ring_index(int v) { return v; }
+constexpr int gcd_of(int a, int b) { return b == 0 ? a : gcd_of(b, a % b); }
+
 // Compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>).  The
 // pipeline body is laid out slot by slot with every index a constant; this does not lean
 // on the loop unroller, whose failure would turn the accumulators into scratch memory.
@@ -90,18 +97,18 @@ __device__ __forceinline__ void static_for(F &&f) {
 // LDS operand read and its wait, written as assembly: the optimiser moves ordinary LDS loads
 // freely (it batched them at the top of the loop, which both breaks the interleave with
 // the MFMAs and blows the register budget), so the reads are pinned here and the kernel
-// does its own lgkmcnt accounting.  lds_wait_all ties the fragment registers through the
-// wait so no MFMA that consumes them can be scheduled above it.
+// does its own lgkmcnt accounting.
 template <int OFFSET>
 __device__ __forceinline__ half8 lds_read16(uint32_t addr) {
     half8 v;
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFFSET));
     return v;
 }
-__device__ __forceinline__ void lds_wait_all(half8 &a, half8 &b, half8 &c, half8 &d) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
-}
-__device__ __forceinline__ void lds_wait_all(half8 &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a)); }
+__device__ __forceinline__ void lds_wait_all() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// Ordered no-op that "modifies" a fragment: placed after lds_wait_all, it keeps every later
+// use of the fragment (the MFMAs, or a register copy the compiler makes) behind the wait
+// without spending an instruction per fragment.
+__device__ __forceinline__ void lds_landed(half8 &a) { asm volatile("" : "+v"(a)); }
 
 // The MFMA itself is issued from assembly too, with the accumulator pinned to AGPRs: that
 // fixes the order of MFMAs, operand reads and copies exactly as written (volatile
@@ -127,6 +134,30 @@ struct MfmaOp<16> {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
+
+// One MFMA slot that also starts a direct-to-LDS copy: M0 (the LDS destination) is set
+// before the MFMA, which doubles as the wait state the hardware wants between a write of
+// M0 and the copy that reads it, so the slot costs three instructions.
+template <int MI, int LDS_IMM>
+__device__ __forceinline__ void mfma_and_dma(half8 a, half8 b, typename MfmaOp<MI>::Acc &c, const void *sbase,
+                                             uint32_t voff, uint32_t lds_base) {
+    if constexpr (MI == 16)
+        asm volatile(
+            "s_add_u32 m0, %3, %6\n\t"
+            "v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\t"
+            "global_load_lds_dwordx4 %4, %5"
+            : "+a"(c)
+            : "v"(a), "v"(b), "s"(lds_base), "v"(voff), "s"(sbase), "i"(LDS_IMM)
+            : "memory", "scc");
+    else
+        asm volatile(
+            "s_add_u32 m0, %3, %6\n\t"
+            "v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\t"
+            "global_load_lds_dwordx4 %4, %5"
+            : "+a"(c)
+            : "v"(a), "v"(b), "s"(lds_base), "v"(voff), "s"(sbase), "i"(LDS_IMM)
+            : "memory", "scc");
+}
 
 // Ordered no-op that "modifies" an accumulator: later reads of it stay behind this point.
 template <class Acc>
@@ -314,13 +345,10 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     // every outstanding operand read has landed; ties all fragments of buffer `buf`
     auto wait_operands = [&](auto buf_c) {
         constexpr int buf = decltype(buf_c)::value;
-        static_for<TM / 4>([&](auto g) {
-            constexpr int t = decltype(g)::value * 4;
-            lds_wait_all(a_frag[buf][t], a_frag[buf][t + 1], a_frag[buf][t + 2], a_frag[buf][t + 3]);
-        });
-        static_for<TM % 4>([&](auto r) { lds_wait_all(a_frag[buf][TM / 4 * 4 + decltype(r)::value]); });
-        static_for<NSB>([&](auto t) { lds_wait_all(b_frag[decltype(t)::value]); });
-        static_for<NDB>([&](auto t) { lds_wait_all(b_last[buf][decltype(t)::value]); });
+        lds_wait_all();
+        static_for<TM>([&](auto t) { lds_landed(a_frag[buf][decltype(t)::value]); });
+        static_for<NSB>([&](auto t) { lds_landed(b_frag[decltype(t)::value]); });
+        static_for<NDB>([&](auto t) { lds_landed(b_last[buf][decltype(t)::value]); });
     };
 
     Acc acc[TM][TN];
@@ -339,6 +367,19 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             MfmaOp<MI>::run(b_last[fb][j - NSB], a_frag[fb][i], acc[i][j]);
         else
             MfmaOp<MI>::run(b_frag[j], a_frag[fb][i], acc[i][j]);
+    };
+    // the same slot, also issuing copy instruction d of the chunk being fetched
+    auto mma_and_copy = [&](auto idx_c, auto fb_c, auto d_c, const unsigned char *a_src, const unsigned char *b_src,
+                            uint32_t dst_a, uint32_t dst_b) {
+        constexpr int idx = decltype(idx_c)::value, fb = decltype(fb_c)::value, d = decltype(d_c)::value;
+        constexpr int j = idx / TM, i = idx % TM;
+        constexpr int imm = (d < A_DMA ? d : d - A_DMA) * Cfg::WAVES * 1024;
+        const unsigned char *src = d < A_DMA ? a_src : b_src;
+        const uint32_t dst = d < A_DMA ? dst_a : dst_b;
+        if constexpr (j >= NSB)
+            mfma_and_dma<MI, imm>(b_last[fb][j - NSB], a_frag[fb][i], acc[i][j], src, voff[d], dst);
+        else
+            mfma_and_dma<MI, imm>(b_frag[j], a_frag[fb][i], acc[i][j], src, voff[d], dst);
     };
 
     // ---- pipeline.  Chunk c of A lives in A-ring buffer c % SA, of B in B-ring buffer c % SB.
@@ -366,6 +407,12 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             return d < A_DMA ? d * LAST0 / A_DMA + 5 : LAST0 + (d - A_DMA) * NMMA / B_DMA + 3;
         return LAST0 + d * NMMA / L;
     };
+    // copy instruction issued in slot `slot`, or -1 (no two copies share a slot)
+    auto copy_in_slot = [copy_slot](int slot) constexpr -> int {
+        for (int d = 0; d < L; ++d)
+            if (copy_slot(d) == slot) return d;
+        return -1;
+    };
     // copies of this iteration issued before its barrier (the barrier opens the last step)
     constexpr int D_BEFORE = SPREAD ? (LAST0 * L + KSTEPS * NMMA - 1) / (KSTEPS * NMMA) : (DEEP_A ? A_DMA : 0);
     // copies allowed to be still in flight at the barrier while chunk kt+1 must have landed
@@ -392,15 +439,26 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     });
     wait_operands(std::integral_constant<int, 0>{});
 
+    const unsigned char *a_next = a_base + AHEAD * BK * 2, *b_next = b_base + AHEAD * BK * 2;
     // One iteration = one K chunk.  ISSUE: chunk kt+AHEAD exists and is copied now.
     // NEXT: chunk kt+1 exists (the barrier is needed and its operands are prefetched).
-    auto iteration = [&](int kt, int cur_a, int cur_b, auto issue_tag, auto next_tag) {
+    // cur_a / cur_b (ring buffers holding chunk kt) are plain ints or, in the unrolled steady
+    // state, compile-time constants: then every LDS address below is a constant offset.
+    auto iteration = [&](int kt, auto cur_a_arg, auto cur_b_arg, auto issue_tag, auto next_tag) {
         constexpr bool ISSUE = decltype(issue_tag)::value, NEXT = decltype(next_tag)::value;
+        const int cur_a = ring_index(cur_a_arg), cur_b = ring_index(cur_b_arg);
         const int nxt_a = (cur_a + 1 == SA) ? 0 : cur_a + 1;
         const int nxt_b = (cur_b + 1 == SB) ? 0 : cur_b + 1;
         const int fill_a = (cur_a + FILL_OFF_A) % SA, fill_b = (cur_b + FILL_OFF_B) % SB;
-        const int kbyte = (Cfg::DBG == 2 ? (kt & 1) : (kt + AHEAD)) * BK * 2;
-        const unsigned char *a_src = a_base + kbyte, *b_src = b_base + kbyte;
+        const unsigned char *a_src = a_next, *b_src = b_next;  // chunk kt + AHEAD
+        if constexpr (Cfg::DBG == 2) {
+            a_src = a_base + (kt & 1) * BK * 2;
+            b_src = b_base + (kt & 1) * BK * 2;
+        }
+        if constexpr (ISSUE) {
+            a_next += BK * 2;
+            b_next += BK * 2;
+        }
         const uint32_t dst_a = cp_lds + fill_a * A_BYTES, dst_b = cp_lds + B_REGION + fill_b * B_BYTES;
         static_for<KSTEPS>([&](auto kk_c) {
             constexpr int kk = decltype(kk_c)::value;
@@ -422,7 +480,12 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             using SrcKK = std::integral_constant<int, (last ? 0 : kk + 1)>;
             static_for<NMMA>([&](auto idx_c) {
                 constexpr int idx = decltype(idx_c)::value;
-                mma_one(idx_c, std::integral_constant<int, fb>{});
+                constexpr int copy = (ISSUE && Cfg::DBG != 1 && Cfg::DBG != 4) ? copy_in_slot(kk * NMMA + idx) : -1;
+                if constexpr (copy >= 0)
+                    mma_and_copy(idx_c, std::integral_constant<int, fb>{}, std::integral_constant<int, copy>{}, a_src,
+                                 b_src, dst_a, dst_b);
+                else
+                    mma_one(idx_c, std::integral_constant<int, fb>{});
                 if constexpr (prefetch && Cfg::DBG != 4) {
                     // One operand read per slot at most, spread out (an LDS read in the slot
                     // right after another one stalls MFMA issue): A tile t for the next step
@@ -437,12 +500,6 @@ __global__ void __launch_bounds__(Cfg::THREADS)
                     if constexpr (idx >= TM + RS && (idx - RS) % TM == 0 && (idx - RS) / TM - 1 < NSB)
                         b_frag[(idx - RS) / TM - 1] =
                             read_b(std::integral_constant<int, (idx - RS) / TM - 1>{}, src_b, SrcKK{});
-                }
-                if constexpr (ISSUE && Cfg::DBG != 1 && Cfg::DBG != 4) {
-                    static_for<L>([&](auto d_c) {
-                        if constexpr (copy_slot(decltype(d_c)::value) == kk * NMMA + idx)
-                            dma_one(d_c, a_src, b_src, dst_a, dst_b);
-                    });
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -459,7 +516,16 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     using T = std::true_type;
     using F = std::false_type;
 
-    int kt = 0, cur_a = 0, cur_b = 0;
+    // Steady state, unrolled over one period of the two rings so that the ring indices are
+    // constants: no index arithmetic or address computation is left inside the loop.
+    constexpr int PERIOD = SA * SB / gcd_of(SA, SB);
+    int kt = 0;
+    for (; kt + PERIOD <= num_k - AHEAD; kt += PERIOD)
+        static_for<PERIOD>([&](auto u_c) {
+            constexpr int u = decltype(u_c)::value;
+            iteration(kt + u, std::integral_constant<int, u % SA>{}, std::integral_constant<int, u % SB>{}, T{}, T{});
+        });
+    int cur_a = 0, cur_b = 0;  // kt is a multiple of the period here
     auto advance = [&] {
         cur_a = (cur_a + 1 == SA) ? 0 : cur_a + 1;
         cur_b = (cur_b + 1 == SB) ? 0 : cur_b + 1;
