@@ -102,7 +102,7 @@ void launch_pipelined_plan(const void *A, const void *B, void *C, size_t M, size
 
 // ---- cost model for the tile-aligned shapes.  A candidate is a tile (its kernel), how
 // many of its workgroups a CU holds, and three times in microseconds fitted to
-// measurements on an MI355X over ~50 shapes (rms error 6 %): `fix` per workgroup
+// measurements on an MI355X over ~45 shapes (rms error 7 %): `fix` per workgroup
 // (prologue, epilogue, scheduling) and the time of one 64-wide K chunk with few (`lo`)
 // and with all (`hi`) CUs busy -- the chip is power-limited, so a chunk costs more when
 // the whole chip computes.  time = launch + full rounds * (fix + chunks * hi)
@@ -113,14 +113,14 @@ struct Candidate {
     double fix, lo, hi;
 };
 constexpr Candidate CANDIDATES[] = {
-    {KERNEL_BIG256, 256, 256, 1, 2, 7.53, 0.978, 1.583},
-    {KERNEL_T192, 192, 192, 1, 3, 4.80, 0.605, 1.045},
-    {KERNEL_R256x128, 256, 128, 1, 3, 4.23, 0.579, 0.930},
-    {KERNEL_MID128, 128, 128, 1, 5, 3.29, 0.350, 0.551},
-    {KERNEL_SMALL64, 64, 64, 3, 3, 1.56, 0.398, 0.611},
+    {KERNEL_BIG256, 256, 256, 1, 2, 7.89, 0.841, 1.490},
+    {KERNEL_T192, 192, 192, 1, 3, 5.10, 0.496, 0.956},
+    {KERNEL_R256x128, 256, 128, 1, 3, 4.29, 0.475, 0.860},
+    {KERNEL_MID128, 128, 128, 1, 5, 3.21, 0.266, 0.510},
+    {KERNEL_SMALL64, 64, 64, 3, 3, 1.41, 0.294, 0.584},
 };
 // launch; reduction kernel: fixed + per slice + fp32 partials written and read back
-constexpr double LAUNCH_US = 0.11, REDUCE_US = 2.64, REDUCE_SLICE_US = 0.15, REDUCE_BYTES_PER_US = 7354e3;
+constexpr double LAUNCH_US = 0.13, REDUCE_US = 3.91, REDUCE_SLICE_US = 0.10, REDUCE_BYTES_PER_US = 7102e3;
 constexpr size_t MAX_PARTIAL_BYTES = 512ull << 20;
 constexpr size_t MAX_PADDED_BYTES = 1024ull << 20;
 size_t padded_n(size_t N) { return (N + 7) / 8 * 8; }
