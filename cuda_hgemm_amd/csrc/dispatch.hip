@@ -1,5 +1,6 @@
 // hgemm_skinny and hgemm_auto: shape-driven choice among the tuned kernels.
 #include "../../include/hgemm.h"
+#include "mfma_decode.h"
 #include "mfma_pipelined.h"
 #include "mfma_ragged.h"
 #include "mfma_skinny.h"
@@ -166,6 +167,13 @@ Plan plan_for(size_t M, size_t N, size_t K) {
     Plan p;
     if (M == 0 || N == 0 || K == 0) return p;
     const size_t cus = (size_t)compute_units();
+    if (M <= 8 && decode_supports(M, N, K)) {  // a few rows: one streaming pass over B, no second launch
+        int bn = 16, waves = 1;
+        decode_plan(M, N, K, cus, &bn, &waves);
+        p.kernel = bn == 16 ? KERNEL_DECODE_BN16 : KERNEL_DECODE_BN32;
+        p.splits = waves;
+        return p;
+    }
     if (skinny_supports(M, N, K)) {
         if (M == 128 && N >= 8192 && N % 128 == 0 && Mid128S4::supports(M, N, K)) {
             p.kernel = KERNEL_MID128_S4;
@@ -292,6 +300,8 @@ void run_plan(const Plan &p, const void *A, const void *B, void *C, size_t M, si
         case KERNEL_SPLIT_64x128: launch_splitk<Split64x128>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_SPLIT_128x64: launch_splitk<Split128x64>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_SPLIT_128x128: launch_splitk<Split128x128>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_DECODE_BN16: launch_decode(A, B, C, M, N, K, 16, p.splits); break;
+        case KERNEL_DECODE_BN32: launch_decode(A, B, C, M, N, K, 32, p.splits); break;
         case KERNEL_RAGGED: launch_ragged(A, B, C, M, N, K); break;
         case KERNEL_PADDED: run_padded(A, B, C, M, N, K); break;
         case KERNEL_SIMT:
@@ -339,6 +349,8 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
         case KERNEL_SPLIT_64x128: return "split-K 64x128x64, 4 waves, 4-stage ring";
         case KERNEL_SPLIT_128x64: return "split-K 128x64x64, 4 waves, 4-stage ring";
         case KERNEL_SPLIT_128x128: return "split-K 128x128x64, 4 waves, 4-stage ring";
+        case KERNEL_DECODE_BN16: return "streaming decode, 16 columns per workgroup, one wave per K slice";
+        case KERNEL_DECODE_BN32: return "streaming decode, 32 columns per workgroup, one wave per K slice";
         case KERNEL_RAGGED: return "guarded 128x128x32, 4 waves, any shape";
         case KERNEL_PADDED: return "zero-padded operand copies + pipelined kernel of the padded shape";
         case KERNEL_SIMT: return "scalar fallback";

@@ -20,6 +20,8 @@ enum KernelId {
     KERNEL_T192,        // pipelined 192x192x64, 4 waves, 3-stage ring
     KERNEL_R256x128,    // pipelined 256x128x64, 4 waves, 3-stage ring
     KERNEL_RAGGED,      // guarded 128x128x32 MFMA kernel: any shape
+    KERNEL_DECODE_BN16, // streaming kernel for M <= 8: 16 or 32 columns per workgroup, `splits` waves over K
+    KERNEL_DECODE_BN32,
     KERNEL_PADDED,      // operands copied zero-padded to N % 8 == 0, K % 64 == 0, then the plan for that shape
 };
 
