@@ -71,10 +71,14 @@ def profiler_command(m: int, n: int, k: int, args) -> list[str]:
     return cmd
 
 
-def run_one(cmd: list[str], log_path: str, timeout_s: float) -> int:
+def run_one(cmd: list[str], log_path: str, timeout_s: float, scratch_dir: str | None = None) -> int:
+    """Runs one command with its output in ``log_path``.  ``scratch_dir``: working directory
+    and TMPDIR of the child (rocprofv3 writes temporary files next to where it runs)."""
+    env = dict(os.environ, TMPDIR=scratch_dir) if scratch_dir else None
     with open(log_path, "w") as log:
         try:
-            return subprocess.run(cmd, stdout=log, stderr=subprocess.STDOUT, timeout=timeout_s).returncode
+            return subprocess.run(cmd, stdout=log, stderr=subprocess.STDOUT, timeout=timeout_s, cwd=scratch_dir,
+                                  env=env).returncode
         except subprocess.TimeoutExpired:
             log.write(f"\nkilled after {timeout_s:.0f} s\n")
             return 124
@@ -101,6 +105,7 @@ def main(argv=None) -> int:
         print(f"{DRIVER} is not built: run python -m cuda_hgemm_amd.build", file=sys.stderr)
         return 2
     dims = [int(d) for d in args.dims.split(",") if d] if args.dims else DIMS
+    args.out = os.path.abspath(args.out)
     os.makedirs(args.out, exist_ok=True)
     failed = 0
     for (m, n, k) in shapes(args.sweep, dims):
@@ -109,7 +114,7 @@ def main(argv=None) -> int:
         if rc == 0 and args.profile:
             print(f"rocprofv3 {m} * {n} * {k}", flush=True)
             rc = run_one(profiler_command(m, n, k, args),
-                         os.path.join(args.out, f"rocprof_hgemm_{m}_{n}_{k}.log"), args.timeout)
+                         os.path.join(args.out, f"rocprof_hgemm_{m}_{n}_{k}.log"), args.timeout, scratch_dir="/tmp")
         if rc != 0:
             failed += 1
             print(f"  driver exited with {rc}, see {args.out}/", file=sys.stderr, flush=True)
