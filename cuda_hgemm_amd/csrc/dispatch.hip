@@ -91,7 +91,13 @@ using Rect256x128 = PipeConfig<256, 128, 64, 2, 2, 3, 16>;
 // ordered reduction (the same one the small-M kernel uses), so the result is bit-identical
 // from run to run.
 template <class Cfg>
-void launch_pipelined_plan(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, int splits) {
+void launch_pipelined_plan(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, const Plan &plan) {
+    const int splits = plan.splits;
+    if (plan.tail_splits > 1) {
+        float *partial = splitk_workspace((size_t)plan.tail_splits * plan.tail_tiles * Cfg::BM * Cfg::BN * sizeof(float));
+        launch_pipelined_with_tail<Cfg>(A, B, C, partial, M, N, K, plan.tail_tiles, plan.tail_splits, "hgemm_auto");
+        return;
+    }
     if (splits <= 1) {
         launch_pipelined<Cfg>(A, B, C, M, N, K, "hgemm_auto");
         return;
@@ -103,7 +109,7 @@ void launch_pipelined_plan(const void *A, const void *B, void *C, size_t M, size
 
 // ---- cost model for the tile-aligned shapes.  A candidate is a tile (its kernel), how
 // many of its workgroups a CU holds, and three times in microseconds fitted to
-// measurements on an MI355X over ~45 shapes (rms error 7 %): `fix` per workgroup
+// measurements on an MI355X over ~55 shapes (rms error 7 %): `fix` per workgroup
 // (prologue, epilogue, scheduling) and the time of one 64-wide K chunk with few (`lo`)
 // and with all (`hi`) CUs busy -- the chip is power-limited, so a chunk costs more when
 // the whole chip computes.  time = launch + full rounds * (fix + chunks * hi)
@@ -114,14 +120,15 @@ struct Candidate {
     double fix, lo, hi;
 };
 constexpr Candidate CANDIDATES[] = {
-    {KERNEL_BIG256, 256, 256, 1, 2, 7.89, 0.841, 1.490},
-    {KERNEL_T192, 192, 192, 1, 3, 5.10, 0.496, 0.956},
-    {KERNEL_R256x128, 256, 128, 1, 3, 4.29, 0.475, 0.860},
-    {KERNEL_MID128, 128, 128, 1, 5, 3.21, 0.266, 0.510},
-    {KERNEL_SMALL64, 64, 64, 3, 3, 1.41, 0.294, 0.584},
+    {KERNEL_BIG256, 256, 256, 1, 2, 7.91, 0.842, 1.463},
+    {KERNEL_T192, 192, 192, 1, 3, 5.11, 0.497, 0.943},
+    {KERNEL_R256x128, 256, 128, 1, 3, 4.25, 0.477, 0.854},
+    {KERNEL_MID128, 128, 128, 1, 5, 3.17, 0.266, 0.510},
+    {KERNEL_SMALL64, 64, 64, 3, 3, 1.38, 0.294, 0.584},
 };
 // launch; reduction kernel: fixed + per slice + fp32 partials written and read back
-constexpr double LAUNCH_US = 0.13, REDUCE_US = 3.91, REDUCE_SLICE_US = 0.10, REDUCE_BYTES_PER_US = 7102e3;
+constexpr double LAUNCH_US = 0.17, REDUCE_US = 3.89, REDUCE_SLICE_US = 0.10, REDUCE_BYTES_PER_US = 7021e3;
+constexpr double TAIL_US = 5.8;  // extra cost of finishing a grid with a separate launch for its last round
 constexpr size_t MAX_PARTIAL_BYTES = 512ull << 20;
 constexpr size_t MAX_PADDED_BYTES = 1024ull << 20;
 size_t padded_n(size_t N) { return (N + 7) / 8 * 8; }
@@ -141,6 +148,19 @@ double predict_us(const Candidate &c, size_t M, size_t N, size_t K, int splits, 
     if (rem) t += c.fix + chunks * (c.lo + (c.hi - c.lo) * (double)rem / (double)slots);
     if (splits > 1)
         t += REDUCE_US + REDUCE_SLICE_US * splits + (double)splits * (double)M * (double)N * 8.0 / REDUCE_BYTES_PER_US;
+    return t;
+}
+
+// The same grid with its last, partly filled round (`rem` workgroups) run in `ts` K slices
+// so that it fills the chip too: whole rounds, then one round of rem * ts shorter
+// workgroups, then the reduction of their compact fp32 partial sums.
+double predict_tail_us(const Candidate &c, size_t M, size_t N, size_t K, int ts, size_t cus) {
+    const size_t wgs = div_ceil(M, (size_t)c.bm) * div_ceil(N, (size_t)c.bn), slots = cus * (size_t)c.per_cu;
+    const size_t full = wgs / slots, rem = wgs % slots;
+    const double chunks = (double)(K / 64);
+    double t = LAUNCH_US + (double)full * (c.fix + chunks * c.hi);
+    t += LAUNCH_US + c.fix + chunks / ts * (c.lo + (c.hi - c.lo) * (double)(rem * ts) / (double)slots);
+    t += REDUCE_US + REDUCE_SLICE_US * ts + (double)ts * (double)rem * c.bm * c.bn * 8.0 / REDUCE_BYTES_PER_US + TAIL_US;
     return t;
 }
 
@@ -203,6 +223,26 @@ Plan plan_for(size_t M, size_t N, size_t K) {
                 p.kernel = c.kernel;
                 p.splits = s;
                 p.est_us = t;
+                p.tail_tiles = 0;
+                p.tail_splits = 1;
+            }
+        }
+        // a grid of whole rounds plus a few workgroups: run those few in K slices
+        const size_t wgs = div_ceil(M, (size_t)c.bm) * div_ceil(N, (size_t)c.bn), slots = cus * (size_t)c.per_cu;
+        const size_t rem = wgs % slots;
+        if (wgs > slots && rem > 0) {
+            for (int ts = 2; ts <= 16; ts *= 2) {
+                if (K % ((size_t)ts * 64) || K / ts < (size_t)64 * c.stages || rem * ts > slots) break;
+                if ((size_t)ts * rem * c.bm * c.bn * sizeof(float) > MAX_PARTIAL_BYTES) break;
+                const double t = predict_tail_us(c, M, N, K, ts, cus);
+                if (p.kernel != KERNEL_NONE && t < best) {
+                    best = t;
+                    p.kernel = c.kernel;
+                    p.splits = 1;
+                    p.est_us = t;
+                    p.tail_tiles = (int)rem;
+                    p.tail_splits = ts;
+                }
             }
         }
     }
@@ -289,12 +329,12 @@ void run_padded(const void *A, const void *B, void *C, size_t M, size_t N, size_
 
 void run_plan(const Plan &p, const void *A, const void *B, void *C, size_t M, size_t N, size_t K) {
     switch (p.kernel) {
-        case KERNEL_BIG256: launch_pipelined_plan<Big256>(A, B, C, M, N, K, p.splits); break;
-        case KERNEL_T192: launch_pipelined_plan<Tile192>(A, B, C, M, N, K, p.splits); break;
-        case KERNEL_R256x128: launch_pipelined_plan<Rect256x128>(A, B, C, M, N, K, p.splits); break;
-        case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_BIG256: launch_pipelined_plan<Big256>(A, B, C, M, N, K, p); break;
+        case KERNEL_T192: launch_pipelined_plan<Tile192>(A, B, C, M, N, K, p); break;
+        case KERNEL_R256x128: launch_pipelined_plan<Rect256x128>(A, B, C, M, N, K, p); break;
+        case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p); break;
         case KERNEL_MID128_S4: launch_pipelined<Mid128S4>(A, B, C, M, N, K, "hgemm_auto"); break;
-        case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p); break;
         case KERNEL_SPLIT_32x64: launch_splitk<Split32x64>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_SPLIT_64x64: launch_splitk<Split64x64>(A, B, C, M, N, K, p.splits); break;
         case KERNEL_SPLIT_64x128: launch_splitk<Split64x128>(A, B, C, M, N, K, p.splits); break;
@@ -335,6 +375,13 @@ extern "C" int hgemm_auto_plan(size_t M, size_t N, size_t K, int *splits) {
     const Plan p = plan_for(M, N, K);
     if (splits) *splits = p.splits;
     return p.kernel;
+}
+// How hgemm_auto treats the last, partly filled round of a large grid: the number of
+// workgroups in it that run in K slices (0: none) and, through `splits`, the slice count.
+extern "C" int hgemm_auto_plan_tail(size_t M, size_t N, size_t K, int *splits) {
+    const Plan p = plan_for(M, N, K);
+    if (splits) *splits = p.tail_splits;
+    return p.tail_tiles;
 }
 extern "C" const char *hgemm_kernel_name(int kernel) {
     switch (kernel) {

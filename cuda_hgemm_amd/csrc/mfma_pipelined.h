@@ -230,7 +230,7 @@ template <class Cfg, bool SPLIT = false, bool EDGE = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_pipelined_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
                            float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n,
-                           long long *trace) {
+                           int first_block, int tail_tiles, long long *trace) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
     constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS, CPR = Cfg::CPR, CPS = Cfg::CPS;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES, SA = Cfg::SA, SB = Cfg::SB;
@@ -252,7 +252,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
 
     int tile_m, tile_n;
-    tile_of_block<Cfg>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_block<Cfg>(first_block + (int)blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
     const int num_k = k_len / BK;
     const int k_begin = SPLIT ? (int)blockIdx.y * k_len : 0;
 
@@ -556,14 +556,25 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     if constexpr (SPLIT) {
         // a lane holds four consecutive n of row m = lane % 16 of each 16x16 tile: 16 bytes of fp32
         const int row = tile_m * BM + wm * Cfg::WM + lane % MI, col = tile_n * BN + wn * Cfg::WN + (lane / MI) * 4;
-        float *dst = partial + ((size_t)blockIdx.y * M + row) * N + col;
-        static_for<TM>([&](auto i_c) {
-            static_for<TN>([&](auto j_c) {
-                constexpr int i = decltype(i_c)::value, j = decltype(j_c)::value;
-                if (!EDGE || (row + i * MI < M && col + j * MI < N))
-                    *reinterpret_cast<floatx4 *>(dst + (size_t)(i * MI) * N + j * MI) = acc[i][j];
+        if (tail_tiles > 0) {  // compact: whole tiles, nothing to guard
+            float *dst = partial + ((size_t)blockIdx.y * tail_tiles + blockIdx.x) * (BM * BN) +
+                         (wm * Cfg::WM + lane % MI) * BN + wn * Cfg::WN + (lane / MI) * 4;
+            static_for<TM>([&](auto i_c) {
+                static_for<TN>([&](auto j_c) {
+                    constexpr int i = decltype(i_c)::value, j = decltype(j_c)::value;
+                    *reinterpret_cast<floatx4 *>(dst + (i * MI) * BN + j * MI) = acc[i][j];
+                });
             });
-        });
+        } else {
+            float *dst = partial + ((size_t)blockIdx.y * M + row) * N + col;
+            static_for<TM>([&](auto i_c) {
+                static_for<TN>([&](auto j_c) {
+                    constexpr int i = decltype(i_c)::value, j = decltype(j_c)::value;
+                    if (!EDGE || (row + i * MI < M && col + j * MI < N))
+                        *reinterpret_cast<floatx4 *>(dst + (size_t)(i * MI) * N + j * MI) = acc[i][j];
+                });
+            });
+        }
     } else {
         (void)partial;
         __syncthreads();
@@ -590,9 +601,43 @@ bool pipelined_supports_edges(size_t M, size_t N, size_t K) {
     return M > 0 && N > 0 && N % 8 == 0 && K % Cfg::BK == 0 && K >= (size_t)Cfg::BK * Cfg::STAGES;
 }
 
+// C[tile of workgroup id first_block + t] = fp16(sum over slices of partial[slice][t][BM][BN]),
+// slices added in order; rows and 8-column pieces outside the matrix are skipped.
+template <class Cfg>
+__global__ void __launch_bounds__(256)
+    tail_reduce_kernel(const float *__restrict__ partial, half_t *__restrict__ C, int M, int N, int tiles_m, int tiles_n,
+                       int first_block, int tail_tiles, int splits) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, PIECES = BM * BN / 8;
+    const int t = blockIdx.y;
+    int tile_m, tile_n;
+    tile_of_block<Cfg>(first_block + t, tiles_m, tiles_n, tile_m, tile_n);
+    const size_t slice_stride = (size_t)tail_tiles * (BM * BN);
+    for (int piece = blockIdx.x * blockDim.x + threadIdx.x; piece < PIECES; piece += gridDim.x * blockDim.x) {
+        const int r = piece / (BN / 8), c = (piece % (BN / 8)) * 8;
+        const int row = tile_m * BM + r, col = tile_n * BN + c;
+        if (row >= M || col >= N) continue;
+        const float *src = partial + (size_t)t * (BM * BN) + r * BN + c;
+        floatx4 s0 = *reinterpret_cast<const floatx4 *>(src);
+        floatx4 s1 = *reinterpret_cast<const floatx4 *>(src + 4);
+        for (int sl = 1; sl < splits; ++sl) {
+            s0 += *reinterpret_cast<const floatx4 *>(src + sl * slice_stride);
+            s1 += *reinterpret_cast<const floatx4 *>(src + sl * slice_stride + 4);
+        }
+        half8 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[e] = (half_t)s0[e];
+            v[4 + e] = (half_t)s1[e];
+        }
+        *reinterpret_cast<half8 *>(C + (size_t)row * N + col) = v;
+    }
+}
+
+// Launches workgroup ids [first_block, first_block + blocks) of the tile grid; tail_tiles
+// as in the kernel.
 template <class Cfg, bool SPLIT, bool EDGE>
 void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial, size_t M, size_t N, size_t K,
-                           int splits, long long *trace) {
+                           int splits, long long *trace, int first_block = 0, int blocks = -1, int tail_tiles = 0) {
     static bool configured = [] {
         HGEMM_CHECK_HIP_ERROR(
             hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg, SPLIT, EDGE>),
@@ -601,10 +646,40 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
     }();
     (void)configured;
     const int tiles_m = (int)div_ceil(M, (size_t)Cfg::BM), tiles_n = (int)div_ceil(N, (size_t)Cfg::BN);
-    hgemm_pipelined_kernel<Cfg, SPLIT, EDGE>
-        <<<dim3(tiles_m * tiles_n, splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
-            reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
-            partial, (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, trace);
+    if (blocks < 0) blocks = tiles_m * tiles_n - first_block;
+    HGEMM_CHECK(first_block >= 0 && blocks >= 1 && first_block + blocks <= tiles_m * tiles_n);
+    hgemm_pipelined_kernel<Cfg, SPLIT, EDGE><<<dim3(blocks, splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
+        reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), partial,
+        (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, first_block, tail_tiles, trace);
+    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+}
+
+// Whole rounds of workgroups computed tile by tile, the last `tail_tiles` workgroup ids in
+// `tail_splits` K slices (so that they fill the chip as well) with an ordered reduction:
+// for grids that end in a nearly empty round.  `partial` holds
+// tail_splits * tail_tiles * BM * BN floats.
+template <class Cfg>
+void launch_pipelined_with_tail(const void *A, const void *B, void *C, float *partial, size_t M, size_t N, size_t K,
+                                int tail_tiles, int tail_splits, const char *name) {
+    check_operands(A, B, C, M, N, K);
+    const int tiles_m = (int)div_ceil(M, (size_t)Cfg::BM), tiles_n = (int)div_ceil(N, (size_t)Cfg::BN);
+    const int total = tiles_m * tiles_n, head = total - tail_tiles;
+    HGEMM_CHECK(partial != nullptr && tail_tiles >= 1 && head >= 1 && tail_splits >= 2 && K % (size_t)tail_splits == 0);
+    HGEMM_CHECK_MSG(pipelined_supports_edges<Cfg>(M, N, K / (size_t)tail_splits),
+                    "%s (tail in %d K slices) needs N %% 8 == 0, slice %% %d == 0, slice >= %d (got M=%zu N=%zu K=%zu)",
+                    name, tail_splits, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
+    if (Cfg::supports(M, N, K)) {
+        launch_pipelined_impl<Cfg, false, false>(A, B, C, nullptr, M, N, K, 1, nullptr, 0, head);
+        launch_pipelined_impl<Cfg, true, false>(A, B, nullptr, partial, M, N, K, tail_splits, nullptr, head, tail_tiles,
+                                                tail_tiles);
+    } else {
+        launch_pipelined_impl<Cfg, false, true>(A, B, C, nullptr, M, N, K, 1, nullptr, 0, head);
+        launch_pipelined_impl<Cfg, true, true>(A, B, nullptr, partial, M, N, K, tail_splits, nullptr, head, tail_tiles,
+                                               tail_tiles);
+    }
+    constexpr int PIECES = Cfg::BM * Cfg::BN / 8;
+    tail_reduce_kernel<Cfg><<<dim3(PIECES / 256 > 8 ? 8 : (PIECES + 255) / 256, tail_tiles), dim3(256), 0, nullptr>>>(
+        partial, reinterpret_cast<half_t *>(C), (int)M, (int)N, tiles_m, tiles_n, head, tail_tiles, tail_splits);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 

@@ -94,6 +94,10 @@ HGEMM_FUNC(hgemm_auto);
 /* Kernel hgemm_auto would pick for a shape (an id for hgemm_kernel_name) and, through
  * `splits` if not NULL, the number of K slices; no launch happens. */
 int hgemm_auto_plan(size_t M, size_t N, size_t K, int *splits);
+/* For grids of whole rounds of workgroups plus a few: how many workgroups of the last round
+ * hgemm_auto runs in K slices so that they fill the chip too (0: none) and, through
+ * `splits` if not NULL, in how many slices. */
+int hgemm_auto_plan_tail(size_t M, size_t N, size_t K, int *splits);
 const char *hgemm_kernel_name(int kernel);
 
 /* ---- registry, so a driver can enumerate variants the way the reference's main lists

@@ -185,6 +185,25 @@ def test_auto_every_tile_with_and_without_k_slices(oracle, hgemm_lib, gpu, shape
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), ref)
 
 
+@pytest.mark.parametrize("shape", [(7168, 7168, 2048), (4352, 4344, 4096), (4352, 4352, 8192)])
+def test_auto_last_round_in_k_slices(oracle, hgemm_lib, gpu, shape):
+    """Grids of whole rounds of workgroups plus a few: the few run in K slices with compact
+    partial sums (also with a ragged N edge).  Complete rows are checked, including rows of
+    the tiles computed in slices."""
+    M, N, K = shape
+    plan = hgemm_lib.auto_plan(M, N, K)
+    assert plan["tail_tiles"] > 0 and plan["tail_splits"] > 1, plan
+    A, B = oracle.fill((M, K), 41, 1), oracle.fill((N, K), 41, 2)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    _sampled_check(oracle, first, A, B, K, rows_per_slab=16, slabs=12, seed=3)
+    assert np.array_equal(first, second)
+    At, Bt = oracle.fill((M, K), 42, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 42, 2, oracle.TERNARY, 0, 1)
+    got = _run(hgemm_lib, "hgemm_auto", At, Bt, gpu)
+    for m0 in range(0, M - 64, 509):          # exact, rows spread over every row of tiles
+        assert np.array_equal(got[m0:m0 + 8], oracle.hgemm_rows(At, Bt, m0, 8)), m0
+    assert np.array_equal(got[M - 8:], oracle.hgemm_rows(At, Bt, M - 8, 8))
+
+
 @pytest.mark.parametrize("N", [4096, 28672])
 @pytest.mark.parametrize("M", [1, 8, 16, 64, 128])
 def test_decode_shapes(oracle, hgemm_lib, gpu, M, N):
