@@ -114,17 +114,18 @@ def main():
     C = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
     auto = lib.variant_fn("hgemm_auto")
 
+    # Order of the reference's driver: the vendor GEMM is evaluated first (src/main.cu:100), the
+    # kernels under test after it.  The part is power-managed and settles only after some tens
+    # of launches, so both are timed twice, alternating, and every pass is reported.
+    Cv = torch.empty_like(C)
+    vms, _ = _time_ms(torch, lib, vendor.fn(), [A], [B], [Cv], M, N, K, args.warmup, args.steps)
     ms, wall_ms = _time_ms(torch, lib, auto, [A], [B], [C], M, N, K, args.warmup, args.steps)
     tflops = lib.tflops(M, N, K, ms)
     out = C.clone()
-
-    Cv = torch.empty_like(C)
-    vms, _ = _time_ms(torch, lib, vendor.fn(), [A], [B], [Cv], M, N, K, args.warmup, args.steps)
-    vendor_tflops = lib.tflops(M, N, K, vms)
-    # second pass of ours after the vendor run: the order of measurement matters on a
-    # power-managed part, report both
+    vms2, _ = _time_ms(torch, lib, vendor.fn(), [A], [B], [Cv], M, N, K, args.warmup, args.steps)
     ms2, _ = _time_ms(torch, lib, auto, [A], [B], [C], M, N, K, args.warmup, args.steps)
     deterministic = bool(torch.equal(out, C))
+    vendor_tflops = lib.tflops(M, N, K, min(vms, vms2))   # the better of its passes is the 100 % line
 
     plan = lib.auto_plan(M, N, K)
     flops = 2.0 * M * N * K
@@ -142,7 +143,8 @@ def main():
                      "launch_ms": ms, "timer": "hipEvent pair on the null stream around the timed launches"},
         "wall_ms_per_step": wall_ms,
         "second_pass_tflops": lib.tflops(M, N, K, ms2),
-        "vendor": {"library": "hipBLASLt (fp32 compute)", "tflops": vendor_tflops, "ms": vms,
+        "vendor": {"library": "hipBLASLt (fp32 compute)", "tflops": vendor_tflops, "ms": min(vms, vms2),
+                   "first_pass_tflops": lib.tflops(M, N, K, vms), "second_pass_tflops": lib.tflops(M, N, K, vms2),
                    "ours_over_vendor": tflops / vendor_tflops},
         "bit_identical_run_to_run": deterministic,
     }
