@@ -247,7 +247,10 @@ def test_skinny_ragged_M(oracle, hgemm_lib, gpu, M):
 RAGGED = [(100, 100, 100), (1, 7, 5), (3, 17, 33), (257, 129, 33), (640, 384, 192), (192, 320, 4096),
           (300, 304, 64), (130, 250, 1000), (1000, 1000, 1000), (129, 4096, 512), (1000, 4000, 1024),
           (1030, 520, 2048), (70, 72, 8192), (2100, 2056, 384), (515, 1032, 4100), (260, 1288, 6144),
-          (2047, 2049, 2051), (2050, 2050, 2048), (64, 1023, 1022)]
+          (2047, 2049, 2051), (2050, 2050, 2048), (64, 1023, 1022),
+          # tile-aligned but K shorter than any LDS ring; tall and thin outputs
+          (256, 256, 64), (512, 512, 128), (128, 128, 64), (4096, 64, 1024), (8192, 8, 512), (2048, 16, 4096),
+          (129, 8, 64), (16, 24, 320), (9, 32, 256), (33, 4096, 256)]
 
 
 @pytest.mark.parametrize("shape", RAGGED)
