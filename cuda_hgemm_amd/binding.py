@@ -41,6 +41,7 @@ HELPER_SYMBOLS = [
     "hgemm_auto_plan", "hgemm_auto_plan_tail", "hgemm_kernel_name", "hgemm_variant_count", "hgemm_variant_name", "hgemm_variant_symbol",
     "hgemm_variant_fn", "hgemm_variant_find", "hgemm_variant_supports", "hgemm_variant_in_default_run",
     "hgemm_profile_ms", "hgemm_profile_rotating_ms", "hgemm_tflops", "hgemm_bytes", "hgemm_version",
+    "hgemm_probe_loop",
 ]
 
 
@@ -105,6 +106,8 @@ class HgemmLibrary:
         d.hgemm_tflops.argtypes, d.hgemm_tflops.restype = [_SZ, _SZ, _SZ, C.c_double], C.c_double
         d.hgemm_bytes.argtypes, d.hgemm_bytes.restype = [_SZ, _SZ, _SZ], C.c_double
         d.hgemm_version.argtypes, d.hgemm_version.restype = [], C.c_char_p
+        d.hgemm_probe_loop.argtypes = [_PTR, _PTR, _PTR, _SZ, _SZ, _SZ, C.c_int, _SZ, C.POINTER(C.c_double)]
+        d.hgemm_probe_loop.restype = None
 
     # ---- registry -------------------------------------------------------------------
     def variants(self) -> List[dict]:

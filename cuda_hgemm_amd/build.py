@@ -29,7 +29,7 @@ DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang
 CXXFLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-I" + INCLUDE]
 
 LIB_SOURCES = ["basic_kernels.hip", "ladder_sync.hip", "ladder_async.hip", "ladder_stages.hip", "dispatch.hip",
-               "api.hip"]
+               "probe.hip", "api.hip"]
 VENDOR_SOURCES = ["vendor_hipblaslt.cpp"]
 DRIVER_SOURCES = ["driver/main.cpp"]
 

@@ -51,6 +51,7 @@ int main(int argc, char *argv[]) {
     flags.define("dist_b", "uniform", "distribution of B");
     flags.define("rotate_mb", "0", "cycle over operand sets totalling at least this many MB (HBM-cold timing)");
     flags.define("json", "", "also write the results to this file as JSON");
+    flags.define("probe", "0", "launches of the in-kernel timing probe of the tuned kernel (0: off; needs M, N % 256 == 0)");
     flags.parse(argc, argv);
 
     const size_t M = flags.u64("M"), N = flags.u64("N"), K = flags.u64("K");
@@ -116,6 +117,8 @@ int main(int argc, char *argv[]) {
             tester.evaluate(hgemm_variant_fn(i), hgemm_variant_name(i));
         }
     }
+
+    if (flags.u64("probe") > 0) tester.probe(flags.u64("probe"));
 
     if (!flags.str("json").empty()) write_json(flags.str("json"), tester, M, N, K, prop);
 

@@ -132,6 +132,17 @@ double hgemm_tflops(size_t M, size_t N, size_t K, double ms);
 /* Algorithmic bytes of one call: 2*(M*K + K*N + M*N). */
 double hgemm_bytes(size_t M, size_t N, size_t K);
 
+/* In-kernel timing of the tuned 256x256x64 kernel (M % 256 == N % 256 == 0, K % 64 == 0):
+ * `launches` back-to-back launches, per-workgroup timestamps taken in the last one.
+ * mode 0: the real kernel; 1: its loop without global->LDS copies; 2: without copies and
+ * without operand reads (modes 1 and 2 leave garbage in C; they price the copies and the
+ * reads).  out8 = { average ms per launch, ms of the traced launch, prologue us, loop us,
+ * epilogue us (means per workgroup), shader cycles in the loop, shader clock in the loop
+ * in GHz, fraction of the loop's cycles covered by the wave's MFMAs }.  No counterpart in
+ * the reference (its profiling is done with ncu, run_sample.sh:23-27). */
+void hgemm_probe_loop(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K, int mode,
+                      size_t launches, double *out8);
+
 /* Library version string. */
 const char *hgemm_version(void);
 
