@@ -10,8 +10,8 @@ line (never part of the measured path), and the CPU checker timed on a bounded s
 same product on this box's host cores.
 
 ``--sweep`` additionally runs every configuration of the specification (squares
-256...16384, the two FFN rectangles, the decode shapes with rotating operands) and writes
-``gpurun_out/bench_sweep.json``; it is not part of the default run.
+256...16384, the two FFN rectangles, the decode shapes with rotating operands), prints the
+table to stderr and writes it as JSON to ``--sweep-out``; it is not part of the default run.
 """
 import argparse
 import json
@@ -98,6 +98,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sweep", action="store_true", help="also run every configuration of the specification")
+    ap.add_argument("--sweep-out", default=os.path.join(ROOT, "gpurun_out", "bench_sweep.json"),
+                    help="where --sweep writes its table as JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (a GEMM shards over N or M with no "
@@ -157,9 +159,9 @@ def main():
             sys.exit(f"GPU result disagrees with the CPU checker: {chk}")
     if args.sweep:
         from cuda_hgemm_amd import sweep
-        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        os.makedirs(os.path.dirname(os.path.abspath(args.sweep_out)), exist_ok=True)
         report = sweep.run(torch, lib, vendor, warmup=args.warmup, steps=args.steps)
-        with open(os.path.join(ROOT, "gpurun_out", "bench_sweep.json"), "w") as f:
+        with open(args.sweep_out, "w") as f:
             json.dump(report, f, indent=1)
         sweep.print_table(report)
     print(json.dumps(result))
