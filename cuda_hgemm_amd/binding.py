@@ -38,7 +38,7 @@ KERNEL_SYMBOLS = [
     "hgemm_mfma_async_stage3", "hgemm_mfma_async_stage4", "hgemm_skinny", "hgemm_auto",
 ]
 HELPER_SYMBOLS = [
-    "hgemm_auto_plan", "hgemm_auto_plan_tail", "hgemm_kernel_name", "hgemm_variant_count", "hgemm_variant_name", "hgemm_variant_symbol",
+    "hgemm_auto_plan", "hgemm_auto_plan_tail", "hgemm_auto_plan_tail_kernel", "hgemm_kernel_name", "hgemm_variant_count", "hgemm_variant_name", "hgemm_variant_symbol",
     "hgemm_variant_fn", "hgemm_variant_find", "hgemm_variant_supports", "hgemm_variant_in_default_run",
     "hgemm_profile_ms", "hgemm_profile_rotating_ms", "hgemm_tflops", "hgemm_bytes", "hgemm_version",
     "hgemm_probe_loop",
@@ -90,6 +90,7 @@ class HgemmLibrary:
             fn.argtypes, fn.restype = _HGEMM_ARGS, None
         d.hgemm_auto_plan.argtypes, d.hgemm_auto_plan.restype = [_SZ, _SZ, _SZ, C.POINTER(C.c_int)], C.c_int
         d.hgemm_auto_plan_tail.argtypes, d.hgemm_auto_plan_tail.restype = [_SZ, _SZ, _SZ, C.POINTER(C.c_int)], C.c_int
+        d.hgemm_auto_plan_tail_kernel.argtypes, d.hgemm_auto_plan_tail_kernel.restype = [_SZ, _SZ, _SZ], C.c_int
         d.hgemm_kernel_name.argtypes, d.hgemm_kernel_name.restype = [C.c_int], C.c_char_p
         d.hgemm_variant_count.argtypes, d.hgemm_variant_count.restype = [], C.c_int
         d.hgemm_variant_name.argtypes, d.hgemm_variant_name.restype = [C.c_int], C.c_char_p
@@ -133,7 +134,8 @@ class HgemmLibrary:
         tail_splits = C.c_int(1)
         tail_tiles = self.dll.hgemm_auto_plan_tail(M, N, K, C.byref(tail_splits))
         return {"kernel_id": kernel, "kernel": self.dll.hgemm_kernel_name(kernel).decode(), "splits": splits.value,
-                "tail_tiles": tail_tiles, "tail_splits": tail_splits.value}
+                "tail_tiles": tail_tiles, "tail_splits": tail_splits.value,
+                "tail_kernel": self.dll.hgemm_kernel_name(self.dll.hgemm_auto_plan_tail_kernel(M, N, K)).decode()}
 
     def version(self) -> str:
         return self.dll.hgemm_version().decode()

@@ -93,6 +93,20 @@ using Rect256x128 = PipeConfig<256, 128, 64, 2, 2, 3, 16>;
 template <class Cfg>
 void launch_pipelined_plan(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, const Plan &plan) {
     const int splits = plan.splits;
+    if constexpr (Cfg::BM == 256 && Cfg::BN == 256) {
+        switch (plan.tail_kernel) {
+            case KERNEL_R256x128:
+                launch_pipelined_with_subtiles<Cfg, Rect256x128>(A, B, C, M, N, K, plan.tail_tiles, "hgemm_auto");
+                return;
+            case KERNEL_MID128:
+                launch_pipelined_with_subtiles<Cfg, Mid128>(A, B, C, M, N, K, plan.tail_tiles, "hgemm_auto");
+                return;
+            case KERNEL_SMALL64:
+                launch_pipelined_with_subtiles<Cfg, Small64>(A, B, C, M, N, K, plan.tail_tiles, "hgemm_auto");
+                return;
+            default: break;
+        }
+    }
     if (plan.tail_splits > 1) {
         float *partial = splitk_workspace((size_t)plan.tail_splits * plan.tail_tiles * Cfg::BM * Cfg::BN * sizeof(float));
         launch_pipelined_with_tail<Cfg>(A, B, C, partial, M, N, K, plan.tail_tiles, plan.tail_splits, "hgemm_auto");
@@ -109,7 +123,7 @@ void launch_pipelined_plan(const void *A, const void *B, void *C, size_t M, size
 
 // ---- cost model for the tile-aligned shapes.  A candidate is a tile (its kernel), how
 // many of its workgroups a CU holds, and three times in microseconds fitted to
-// measurements on an MI355X over ~55 shapes (rms error 7 %): `fix` per workgroup
+// measurements on an MI355X over ~60 shapes (rms error 7 %): `fix` per workgroup
 // (prologue, epilogue, scheduling) and the time of one 64-wide K chunk with few (`lo`)
 // and with all (`hi`) CUs busy -- the chip is power-limited, so a chunk costs more when
 // the whole chip computes.  time = launch + full rounds * (fix + chunks * hi)
@@ -120,15 +134,16 @@ struct Candidate {
     double fix, lo, hi;
 };
 constexpr Candidate CANDIDATES[] = {
-    {KERNEL_BIG256, 256, 256, 1, 2, 7.91, 0.842, 1.463},
-    {KERNEL_T192, 192, 192, 1, 3, 5.11, 0.497, 0.943},
-    {KERNEL_R256x128, 256, 128, 1, 3, 4.25, 0.477, 0.854},
+    {KERNEL_BIG256, 256, 256, 1, 2, 7.92, 0.841, 1.462},
+    {KERNEL_T192, 192, 192, 1, 3, 5.17, 0.495, 0.948},
+    {KERNEL_R256x128, 256, 128, 1, 3, 4.25, 0.476, 0.856},
     {KERNEL_MID128, 128, 128, 1, 5, 3.17, 0.266, 0.510},
-    {KERNEL_SMALL64, 64, 64, 3, 3, 1.38, 0.294, 0.584},
+    {KERNEL_SMALL64, 64, 64, 3, 3, 1.39, 0.294, 0.585},
 };
 // launch; reduction kernel: fixed + per slice + fp32 partials written and read back
-constexpr double LAUNCH_US = 0.17, REDUCE_US = 3.89, REDUCE_SLICE_US = 0.10, REDUCE_BYTES_PER_US = 7021e3;
-constexpr double TAIL_US = 5.8;  // extra cost of finishing a grid with a separate launch for its last round
+constexpr double LAUNCH_US = 0.16, REDUCE_US = 3.90, REDUCE_SLICE_US = 0.10, REDUCE_BYTES_PER_US = 7040e3;
+// extra cost of finishing a grid with a separate launch for its last round: in K slices / on smaller tiles
+constexpr double TAIL_US = 3.6, TAIL_SUB_US = 4.4;
 constexpr size_t MAX_PARTIAL_BYTES = 512ull << 20;
 constexpr size_t MAX_PADDED_BYTES = 1024ull << 20;
 size_t padded_n(size_t N) { return (N + 7) / 8 * 8; }
@@ -162,6 +177,22 @@ double predict_tail_us(const Candidate &c, size_t M, size_t N, size_t K, int ts,
     t += LAUNCH_US + c.fix + chunks / ts * (c.lo + (c.hi - c.lo) * (double)(rem * ts) / (double)slots);
     t += REDUCE_US + REDUCE_SLICE_US * ts + (double)ts * (double)rem * c.bm * c.bn * 8.0 / REDUCE_BYTES_PER_US + TAIL_US;
     return t;
+}
+
+// A grid of 256x256 tiles whose last round (`rem` workgroups) is handed to a smaller tile
+// that divides it: whole rounds of the big tile, then rem * parts workgroups of the small
+// one.  No partial sums and no reduction.
+double predict_subtile_us(const Candidate &big, const Candidate &small, size_t M, size_t N, size_t K, size_t cus) {
+    const size_t wgs = div_ceil(M, (size_t)big.bm) * div_ceil(N, (size_t)big.bn), slots = cus * (size_t)big.per_cu;
+    const size_t full = wgs / slots, rem = wgs % slots;
+    const size_t parts = (size_t)(big.bm / small.bm) * (big.bn / small.bn);
+    const size_t small_slots = cus * (size_t)small.per_cu, small_wgs = rem * parts;
+    const double chunks = (double)(K / 64);
+    double t = LAUNCH_US + (double)full * (big.fix + chunks * big.hi);
+    t += LAUNCH_US + (double)(small_wgs / small_slots) * (small.fix + chunks * small.hi);
+    if (small_wgs % small_slots)
+        t += small.fix + chunks * (small.lo + (small.hi - small.lo) * (double)(small_wgs % small_slots) / (double)small_slots);
+    return t + TAIL_SUB_US;
 }
 
 // Number of K slices for `tiles` output tiles: the smallest power of two (<= 16) that
@@ -225,6 +256,7 @@ Plan plan_for(size_t M, size_t N, size_t K) {
                 p.est_us = t;
                 p.tail_tiles = 0;
                 p.tail_splits = 1;
+                p.tail_kernel = KERNEL_NONE;
             }
         }
         // a grid of whole rounds plus a few workgroups: run those few in K slices
@@ -242,6 +274,23 @@ Plan plan_for(size_t M, size_t N, size_t K) {
                     p.est_us = t;
                     p.tail_tiles = (int)rem;
                     p.tail_splits = ts;
+                    p.tail_kernel = KERNEL_NONE;
+                }
+            }
+            if (c.kernel == KERNEL_BIG256) {  // ... or on smaller tiles that divide this one
+                for (const Candidate &small : CANDIDATES) {
+                    if (small.kernel == KERNEL_BIG256 || c.bm % small.bm || c.bn % small.bn) continue;
+                    if (K < (size_t)64 * small.stages) continue;
+                    const double t = predict_subtile_us(c, small, M, N, K, cus);
+                    if (p.kernel != KERNEL_NONE && t < best) {
+                        best = t;
+                        p.kernel = c.kernel;
+                        p.splits = 1;
+                        p.est_us = t;
+                        p.tail_tiles = (int)rem;
+                        p.tail_splits = 1;
+                        p.tail_kernel = small.kernel;
+                    }
                 }
             }
         }
@@ -383,6 +432,8 @@ extern "C" int hgemm_auto_plan_tail(size_t M, size_t N, size_t K, int *splits) {
     if (splits) *splits = p.tail_splits;
     return p.tail_tiles;
 }
+// Kernel id of the smaller tile that takes over the last round (0: none).
+extern "C" int hgemm_auto_plan_tail_kernel(size_t M, size_t N, size_t K) { return plan_for(M, N, K).tail_kernel; }
 extern "C" const char *hgemm_kernel_name(int kernel) {
     switch (kernel) {
         case KERNEL_BIG256: return "pipelined 256x256x64, 4 waves, LDS ring 3 (A) + 2 (B)";

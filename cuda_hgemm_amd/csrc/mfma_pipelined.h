@@ -230,7 +230,7 @@ template <class Cfg, bool SPLIT = false, bool EDGE = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_pipelined_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
                            float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n,
-                           int first_block, int tail_tiles, long long *trace) {
+                           int first_block, int tail_tiles, int subdiv, long long *trace) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
     constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS, CPR = Cfg::CPR, CPS = Cfg::CPS;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES, SA = Cfg::SA, SB = Cfg::SB;
@@ -252,7 +252,19 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
 
     int tile_m, tile_n;
-    tile_of_block<Cfg>(first_block + (int)blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+    if (subdiv == 0) {
+        tile_of_block<Cfg>(first_block + (int)blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+    } else {
+        // tiles_m x tiles_n is the grid of a larger tile that this one divides sub_m x sub_n times;
+        // consecutive workgroups take the parts of workgroup id first_block + blockIdx.x / parts
+        const int sub_m = subdiv >> 8, sub_n = subdiv & 255, parts = sub_m * sub_n;
+        const int part = (int)blockIdx.x % parts;
+        int parent_m, parent_n;
+        tile_of_block<Cfg>(first_block + (int)blockIdx.x / parts, tiles_m, tiles_n, parent_m, parent_n);
+        tile_m = parent_m * sub_m + part / sub_n;
+        tile_n = parent_n * sub_n + part % sub_n;
+        if (tile_m * BM >= M || tile_n * BN >= N) return;  // a part wholly outside the matrix (whole workgroup)
+    }
     const int num_k = k_len / BK;
     const int k_begin = SPLIT ? (int)blockIdx.y * k_len : 0;
 
@@ -638,6 +650,7 @@ __global__ void __launch_bounds__(256)
 template <class Cfg, bool SPLIT, bool EDGE>
 void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial, size_t M, size_t N, size_t K,
                            int splits, long long *trace, int first_block = 0, int blocks = -1, int tail_tiles = 0) {
+    constexpr int subdiv = 0;
     static bool configured = [] {
         HGEMM_CHECK_HIP_ERROR(
             hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg, SPLIT, EDGE>),
@@ -650,7 +663,7 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
     HGEMM_CHECK(first_block >= 0 && blocks >= 1 && first_block + blocks <= tiles_m * tiles_n);
     hgemm_pipelined_kernel<Cfg, SPLIT, EDGE><<<dim3(blocks, splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), partial,
-        (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, first_block, tail_tiles, trace);
+        (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, first_block, tail_tiles, subdiv, trace);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 
@@ -712,6 +725,43 @@ void launch_pipelined_split(const void *A, const void *B, float *partial, size_t
                     "%s (K in %d slices) needs N %% 8 == 0, slice %% %d == 0, slice >= %d (got M=%zu N=%zu K=%zu)",
                     name, splits, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
     launch_pipelined_impl<Cfg, true, true>(A, B, nullptr, partial, M, N, K, splits, nullptr);
+}
+
+// Whole rounds of workgroups on the Parent tile, the last `tail_tiles` workgroup ids of its
+// grid on the smaller Child tile (Parent::BM % Child::BM == 0, likewise BN), each parent tile
+// divided among (Parent::BM / Child::BM) * (Parent::BN / Child::BN) workgroups: no partial
+// sums, no reduction, one more launch.
+template <class Parent, class Child>
+void launch_pipelined_with_subtiles(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, int tail_tiles,
+                                    const char *name) {
+    static_assert(Parent::BM % Child::BM == 0 && Parent::BN % Child::BN == 0 && Parent::GROUP_N == Child::GROUP_N,
+                  "the child tile must divide the parent tile and share its rasterisation");
+    check_operands(A, B, C, M, N, K);
+    constexpr int sub_m = Parent::BM / Child::BM, sub_n = Parent::BN / Child::BN;
+    const int tiles_m = (int)div_ceil(M, (size_t)Parent::BM), tiles_n = (int)div_ceil(N, (size_t)Parent::BN);
+    const int head = tiles_m * tiles_n - tail_tiles;
+    HGEMM_CHECK(tail_tiles >= 1 && head >= 1);
+    HGEMM_CHECK_MSG(pipelined_supports_edges<Parent>(M, N, K) && pipelined_supports_edges<Child>(M, N, K),
+                    "%s needs N %% 8 == 0, K %% 64 == 0, K >= %d (got M=%zu N=%zu K=%zu)", name,
+                    64 * (Parent::STAGES > Child::STAGES ? Parent::STAGES : Child::STAGES), M, N, K);
+    if (Parent::supports(M, N, K))
+        launch_pipelined_impl<Parent, false, false>(A, B, C, nullptr, M, N, K, 1, nullptr, 0, head);
+    else
+        launch_pipelined_impl<Parent, false, true>(A, B, C, nullptr, M, N, K, 1, nullptr, 0, head);
+    const bool edge = !Child::supports(M, N, K);
+    auto kernel = edge ? &hgemm_pipelined_kernel<Child, false, true> : &hgemm_pipelined_kernel<Child, false, false>;
+    static bool configured = [] {
+        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Child, false, true>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, Child::LDS_BYTES));
+        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Child, false, false>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, Child::LDS_BYTES));
+        return true;
+    }();
+    (void)configured;
+    kernel<<<dim3(tail_tiles * sub_m * sub_n), dim3(Child::THREADS), Child::LDS_BYTES, nullptr>>>(
+        reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), nullptr,
+        (int)M, (int)N, (int)K, (int)K, tiles_m, tiles_n, head, 0, (sub_m << 8) | sub_n, nullptr);
+    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 
 }  // namespace hgemm

@@ -29,8 +29,9 @@ struct Plan {
     int kernel = KERNEL_NONE;
     int splits = 1;
     double est_us = 0.0;  // the cost model's estimate where it was used, else 0
-    // pipelined kernels only: the last tail_tiles workgroup ids of the grid run in tail_splits K slices
-    int tail_tiles = 0, tail_splits = 1;
+    // pipelined kernels only: the last tail_tiles workgroup ids of the grid run in tail_splits K slices, or
+    // (tail_kernel != KERNEL_NONE, 256x256 tiles only) divided among workgroups of that smaller tile
+    int tail_tiles = 0, tail_splits = 1, tail_kernel = KERNEL_NONE;
 };
 
 bool skinny_supports(size_t M, size_t N, size_t K);

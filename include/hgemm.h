@@ -98,6 +98,10 @@ int hgemm_auto_plan(size_t M, size_t N, size_t K, int *splits);
  * hgemm_auto runs in K slices so that they fill the chip too (0: none) and, through
  * `splits` if not NULL, in how many slices. */
 int hgemm_auto_plan_tail(size_t M, size_t N, size_t K, int *splits);
+/* The other treatment of such a last round: its workgroups' tiles are divided among
+ * workgroups of a smaller tile.  Returns that kernel's id (for hgemm_kernel_name), 0 if
+ * the plan does not do this; hgemm_auto_plan_tail still gives the number of tiles. */
+int hgemm_auto_plan_tail_kernel(size_t M, size_t N, size_t K);
 const char *hgemm_kernel_name(int kernel);
 
 /* ---- registry, so a driver can enumerate variants the way the reference's main lists

@@ -185,14 +185,20 @@ def test_auto_every_tile_with_and_without_k_slices(oracle, hgemm_lib, gpu, shape
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), ref)
 
 
-@pytest.mark.parametrize("shape", [(7168, 7168, 2048), (4352, 4344, 4096), (4352, 4352, 8192)])
-def test_auto_last_round_in_k_slices(oracle, hgemm_lib, gpu, shape):
+@pytest.mark.parametrize("shape,mode", [((7168, 7168, 7168), "k slices"), ((7168, 7168, 2048), "128x128x64"),
+                                        ((4352, 4344, 4096), "128x128x64"), ((4352, 4352, 1024), "64x64x64"),
+                                        ((4096, 14336, 4096), "256x128x64"), ((4360, 4352, 512), "128x128x64")])
+def test_auto_last_round_of_a_large_grid(oracle, hgemm_lib, gpu, shape, mode):
     """Grids of whole rounds of workgroups plus a few: the few run in K slices with compact
-    partial sums (also with a ragged N edge).  Complete rows are checked, including rows of
-    the tiles computed in slices."""
+    partial sums, or their tiles are divided among workgroups of a smaller tile (also with
+    ragged edges).  Complete rows are checked, including rows of the tiles treated that way."""
     M, N, K = shape
     plan = hgemm_lib.auto_plan(M, N, K)
-    assert plan["tail_tiles"] > 0 and plan["tail_splits"] > 1, plan
+    assert plan["tail_tiles"] > 0, plan
+    if mode == "k slices":
+        assert plan["tail_splits"] > 1 and plan["tail_kernel"] == "none", plan
+    else:
+        assert plan["tail_splits"] == 1 and mode in plan["tail_kernel"], plan
     A, B = oracle.fill((M, K), 41, 1), oracle.fill((N, K), 41, 2)
     first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
     _sampled_check(oracle, first, A, B, K, rows_per_slab=16, slabs=12, seed=3)
