@@ -291,6 +291,45 @@ def test_guarded_edges_do_not_write_outside_c(oracle, hgemm_lib, gpu):
         _assert_close(oracle, host[pad:pad + M * N].reshape(M, N), oracle.hgemm(A, B), K)
 
 
+def test_auto_random_shapes_against_the_vendor_comparator(oracle, hgemm_lib, vendor_lib, gpu):
+    """300 seeded shapes over every alignment class the dispatcher distinguishes (tile
+    multiples, N % 8, K % 64, K % 8, odd everything; small, tall, wide, deep), each against
+    hipBLASLt on the same inputs -- the comparator itself is pinned against the CPU checker
+    above.  Both accumulate in fp32 and round once, so they agree to an output ulp; the
+    specification's tolerance is asserted, plus bit-identity from run to run."""
+    import torch
+    rng = np.random.default_rng(20230212)
+    grains = [(256, 256, 64), (64, 64, 64), (8, 8, 64), (1, 8, 64), (1, 8, 8), (1, 1, 8), (1, 1, 1)]
+    gen = torch.Generator(device=gpu).manual_seed(7)
+    checked = 0
+    for i in range(300):
+        gm, gn, gk = grains[i % len(grains)]
+        big = i % 3 == 0
+        top = 9000 if (big and gm == 256) else (5000 if big else 700)   # the largest reach grids with a last round
+        M = int(rng.integers(1, top // gm + 1)) * gm
+        N = int(rng.integers(1, top // gn + 1)) * gn
+        K = int(rng.integers(1, (3000 if big else 9000) // gk + 1)) * gk
+        if i % 10 == 7:
+            M = int(rng.integers(1, 129))                      # decode-like
+        A = (torch.rand((M, K), device=gpu, generator=gen) * 2 - 1).half()
+        B = (torch.rand((N, K), device=gpu, generator=gen) * 2 - 1).half()
+        C = torch.full((M, N), POISON - 65536, dtype=torch.int16, device=gpu).view(torch.float16)
+        C2 = torch.full((M, N), POISON - 65536, dtype=torch.int16, device=gpu).view(torch.float16)
+        Cv = torch.empty((M, N), dtype=torch.float16, device=gpu)
+        plan = hgemm_lib.auto_plan(M, N, K)
+        print(f"[gpu] hgemm_auto M={M} N={N} K={K} {plan['kernel']} x{plan['splits']} tail {plan['tail_tiles']}",
+              flush=True)
+        hgemm_lib.call("hgemm_auto", A, B, C, M, N, K)
+        hgemm_lib.call("hgemm_auto", A, B, C2, M, N, K)
+        vendor_lib.call(A, B, Cv, M, N, K)
+        got, again, ref = _to_bits(C), _to_bits(C2), _to_bits(Cv)
+        res = oracle.check(got, ref, K)
+        assert res["non_finite"] == 0 and res["ok"], (M, N, K, plan, res)
+        assert np.array_equal(got, again), (M, N, K, plan)
+        checked += 1
+    assert checked == 300
+
+
 # ------------------------------------------------------------------ size-independent properties at full size
 def test_properties_at_8192(oracle, hgemm_lib, gpu):
     import torch
