@@ -10,6 +10,7 @@ back into tables and charts.
     python -m cuda_hgemm_amd.benchmark --sweep wide --out log_wide   # M = N > K
     python -m cuda_hgemm_amd.benchmark --sweep deep --out log_deep   # M = N < K
     python -m cuda_hgemm_amd.benchmark --profile --dims 8192         # under rocprofv3 (the reference: ncu)
+    python -m cuda_hgemm_amd.benchmark --pmc mfma --dims 8192        # hardware counters, one named set per run
 
 The driver is started as a child process per shape, like the shell loop of the reference;
 this module never touches the GPU itself.
@@ -25,6 +26,18 @@ import time
 # the reference's dimension list (run_sample.sh:30)
 DIMS = [256, 512, 768, 1024, 1536, 2048, 3072, 4096, 5120, 6144, 7168, 8192, 9216, 10240, 11264, 12288, 13312,
         14336, 15360, 16384]
+
+# Hardware-counter sets for --pmc, each small enough for one pass (rocprofv3 does not split
+# counters over passes: at most 8 SQ, 4 TCC -- FETCH_SIZE takes 3 of them, WRITE_SIZE 2 -- and
+# 2 GRBM counters per run).  Together they cover what the reference's `ncu --set full` run is
+# read for (run_sample.sh:23-27): matrix-pipe occupancy, LDS bank conflicts, bytes moved
+# between L2 and the memory fabric.
+PMC_SETS = {
+    "mfma": ["SQ_VALU_MFMA_BUSY_CYCLES", "SQ_INSTS_VALU_MFMA_MOPS_F16", "SQ_BUSY_CYCLES", "SQ_WAVES", "GRBM_GUI_ACTIVE"],
+    "lds": ["SQ_LDS_BANK_CONFLICT", "SQ_LDS_IDX_ACTIVE", "SQ_INSTS_LDS", "SQ_VALU_MFMA_BUSY_CYCLES", "GRBM_GUI_ACTIVE"],
+    "fetch": ["FETCH_SIZE"],
+    "write": ["WRITE_SIZE"],
+}
 
 PACKAGE_DIR = os.path.dirname(os.path.abspath(__file__))
 DRIVER = os.path.join(PACKAGE_DIR, "bin", "hgemm")
@@ -58,14 +71,17 @@ def driver_command(m: int, n: int, k: int, args) -> list[str]:
     return cmd
 
 
-def profiler_command(m: int, n: int, k: int, args) -> list[str]:
-    """rocprofv3 kernel trace of one shape with a single timed iteration, in place of the
-    reference's ``ncu --set full`` run (run_sample.sh:23-27).  The driver binary itself
-    follows ``--``: the profiler must not be handed a launcher that re-executes."""
-    out_dir = os.path.join(os.path.abspath(args.out), "rocprof", f"hgemm_{m}_{n}_{k}")
+def profiler_command(m: int, n: int, k: int, args, pmc: str = "") -> list[str]:
+    """rocprofv3 run of one shape with a single timed iteration, in place of the reference's
+    ``ncu --set full`` run (run_sample.sh:23-27): a kernel trace with per-kernel statistics,
+    or -- ``pmc`` names one of PMC_SETS -- hardware counters per dispatch.  Counters and
+    traces never share a run.  The driver binary itself follows ``--``: the profiler must not
+    be handed a launcher that re-executes."""
+    out_dir = os.path.join(os.path.abspath(args.out), "rocprof" + ("_" + pmc if pmc else ""), f"hgemm_{m}_{n}_{k}")
     saved = (args.warmup, args.iterations)
     args.warmup, args.iterations = 1, 1
-    cmd = ["rocprofv3", "--kernel-trace", "--stats", "--output-format", "csv", "-d", out_dir, "-o", "hgemm", "--"]
+    what = ["--pmc"] + PMC_SETS[pmc] if pmc else ["--kernel-trace", "--stats"]
+    cmd = ["rocprofv3"] + what + ["--output-format", "csv", "-d", out_dir, "-o", "hgemm", "--"]
     cmd += driver_command(m, n, k, args)
     args.warmup, args.iterations = saved
     return cmd
@@ -97,6 +113,8 @@ def main(argv=None) -> int:
     ap.add_argument("--variant", default="", help="evaluate only this variant next to hipBLASLt")
     ap.add_argument("--json", action="store_true", help="also keep the driver's JSON report per shape")
     ap.add_argument("--profile", action="store_true", help="additionally trace each shape under rocprofv3")
+    ap.add_argument("--pmc", default="", help="comma-separated counter sets to collect per shape, one rocprofv3 run "
+                    "each: " + ", ".join(f"{k} ({' '.join(v)})" for k, v in PMC_SETS.items()))
     ap.add_argument("--timeout", type=float, default=300.0, help="seconds allowed per driver run")
     ap.add_argument("--pause", type=float, default=0.0, help="seconds between shapes (the reference sleeps 3)")
     args = ap.parse_args(argv)
@@ -105,6 +123,11 @@ def main(argv=None) -> int:
         print(f"{DRIVER} is not built: run python -m cuda_hgemm_amd.build", file=sys.stderr)
         return 2
     dims = [int(d) for d in args.dims.split(",") if d] if args.dims else DIMS
+    pmc_sets = [p for p in args.pmc.split(",") if p]
+    for p in pmc_sets:
+        if p not in PMC_SETS:
+            print(f"unknown counter set '{p}' (known: {', '.join(PMC_SETS)})", file=sys.stderr)
+            return 2
     args.out = os.path.abspath(args.out)
     os.makedirs(args.out, exist_ok=True)
     failed = 0
@@ -115,6 +138,12 @@ def main(argv=None) -> int:
             print(f"rocprofv3 {m} * {n} * {k}", flush=True)
             rc = run_one(profiler_command(m, n, k, args),
                          os.path.join(args.out, f"rocprof_hgemm_{m}_{n}_{k}.log"), args.timeout, scratch_dir="/tmp")
+        for p in pmc_sets if rc == 0 else []:
+            print(f"rocprofv3 --pmc {p} {m} * {n} * {k}", flush=True)
+            rc = run_one(profiler_command(m, n, k, args, pmc=p),
+                         os.path.join(args.out, f"rocprof_{p}_hgemm_{m}_{n}_{k}.log"), args.timeout, scratch_dir="/tmp")
+            if rc != 0:
+                break
         if rc != 0:
             failed += 1
             print(f"  driver exited with {rc}, see {args.out}/", file=sys.stderr, flush=True)

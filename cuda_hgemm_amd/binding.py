@@ -35,13 +35,15 @@ HGEMM_FN = C.CFUNCTYPE(None, *_HGEMM_ARGS)
 KERNEL_SYMBOLS = [
     "hgemm_simt_naive", "hgemm_mfma_naive", "hgemm_mfma_base", "hgemm_mfma_padding", "hgemm_mfma_swizzle",
     "hgemm_mfma_async", "hgemm_mfma_async_pg2s", "hgemm_mfma_async_pg2s_ps2r", "hgemm_mfma_async_stage2",
-    "hgemm_mfma_async_stage3", "hgemm_mfma_async_stage4", "hgemm_skinny", "hgemm_auto",
+    "hgemm_mfma_async_stage3", "hgemm_mfma_async_stage4", "hgemm_mfma_pipelined_64x64",
+    "hgemm_mfma_pipelined_128x128", "hgemm_mfma_pipelined_192x192", "hgemm_mfma_pipelined_256x128",
+    "hgemm_mfma_pipelined_256x256", "hgemm_skinny", "hgemm_auto",
 ]
 HELPER_SYMBOLS = [
     "hgemm_auto_plan", "hgemm_auto_plan_tail", "hgemm_auto_plan_tail_kernel", "hgemm_kernel_name", "hgemm_variant_count", "hgemm_variant_name", "hgemm_variant_symbol",
     "hgemm_variant_fn", "hgemm_variant_find", "hgemm_variant_supports", "hgemm_variant_in_default_run",
     "hgemm_profile_ms", "hgemm_profile_rotating_ms", "hgemm_tflops", "hgemm_bytes", "hgemm_version",
-    "hgemm_probe_loop",
+    "hgemm_reserve_workspace", "hgemm_release_workspace", "hgemm_auto_workspace_bytes",
 ]
 
 
@@ -107,8 +109,10 @@ class HgemmLibrary:
         d.hgemm_tflops.argtypes, d.hgemm_tflops.restype = [_SZ, _SZ, _SZ, C.c_double], C.c_double
         d.hgemm_bytes.argtypes, d.hgemm_bytes.restype = [_SZ, _SZ, _SZ], C.c_double
         d.hgemm_version.argtypes, d.hgemm_version.restype = [], C.c_char_p
-        d.hgemm_probe_loop.argtypes = [_PTR, _PTR, _PTR, _SZ, _SZ, _SZ, C.c_int, _SZ, C.POINTER(C.c_double)]
-        d.hgemm_probe_loop.restype = None
+        d.hgemm_reserve_workspace.argtypes, d.hgemm_reserve_workspace.restype = [_SZ, _SZ], C.c_int
+        d.hgemm_release_workspace.argtypes, d.hgemm_release_workspace.restype = [], None
+        d.hgemm_auto_workspace_bytes.argtypes = [_SZ, _SZ, _SZ, C.POINTER(_SZ)]
+        d.hgemm_auto_workspace_bytes.restype = _SZ
 
     # ---- registry -------------------------------------------------------------------
     def variants(self) -> List[dict]:
@@ -136,6 +140,18 @@ class HgemmLibrary:
         return {"kernel_id": kernel, "kernel": self.dll.hgemm_kernel_name(kernel).decode(), "splits": splits.value,
                 "tail_tiles": tail_tiles, "tail_splits": tail_splits.value,
                 "tail_kernel": self.dll.hgemm_kernel_name(self.dll.hgemm_auto_plan_tail_kernel(M, N, K)).decode()}
+
+    def auto_workspace_bytes(self, M: int, N: int, K: int) -> dict:
+        operands = _SZ(0)
+        partial = self.dll.hgemm_auto_workspace_bytes(M, N, K, C.byref(operands))
+        return {"partial": partial, "operands": operands.value}
+
+    def reserve_workspace(self, partial_bytes: int = 0, operand_bytes: int = 0) -> None:
+        if self.dll.hgemm_reserve_workspace(partial_bytes, operand_bytes) != 0:
+            raise MemoryError("hgemm_reserve_workspace: device memory ran out")
+
+    def release_workspace(self) -> None:
+        self.dll.hgemm_release_workspace()
 
     def version(self) -> str:
         return self.dll.hgemm_version().decode()

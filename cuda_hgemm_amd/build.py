@@ -3,6 +3,7 @@
     cuda_hgemm_amd/lib/libhgemm.so            the kernels + C ABI (include/hgemm.h)
     cuda_hgemm_amd/lib/libhgemm_hipblaslt.so  vendor comparator (include/hgemm_hipblaslt.h)
     cuda_hgemm_amd/bin/hgemm                  C++ benchmark / check driver
+    cuda_hgemm_amd/bin/hgemm_probe            in-kernel timing of the tuned kernel (evidence tool)
 
 Run as ``python -m cuda_hgemm_amd.build`` (add ``--force`` to rebuild everything).
 hipcc cross-compiles without a GPU, so this works on a CPU-only machine.
@@ -29,9 +30,10 @@ DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang
 CXXFLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-I" + INCLUDE]
 
 LIB_SOURCES = ["basic_kernels.hip", "ladder_sync.hip", "ladder_async.hip", "ladder_stages.hip", "dispatch.hip",
-               "probe.hip", "api.hip"]
+               "api.hip"]
 VENDOR_SOURCES = ["vendor_hipblaslt.cpp"]
 DRIVER_SOURCES = ["driver/main.cpp"]
+PROBE_SOURCES = ["probe/probe_loop.hip"]   # bin/hgemm_probe: in-kernel timing, not part of the library
 
 
 def _headers():
@@ -57,21 +59,54 @@ def _run(cmd):
     return "\n".join(lines)
 
 
+# Kernels whose operands and accumulators are handled from inline assembly in an order the
+# compiler does not know: a register spill between an LDS read and its wait, or of an
+# accumulator, would corrupt results silently, so the build fails if one appears.
+NO_SPILL_KERNELS = ("hgemm_pipelined_kernel",)
+
+
+def _check_no_spills(src, remarks):
+    """`remarks`: output of -Rpass-analysis=kernel-resource-usage for one source file."""
+    name, checked = None, 0
+    for line in remarks.splitlines():
+        if "remark: Function Name:" in line:
+            name = line.split("Function Name:")[1].split()[0]
+            continue
+        if name is None or not any(k in name for k in NO_SPILL_KERNELS):
+            continue
+        for key in ("ScratchSize [bytes/lane]:", "SGPRs Spill:", "VGPRs Spill:"):
+            if key in line:
+                value = int(line.split(key)[1].split()[0])
+                checked += 1
+                if value != 0 and key != "SGPRs Spill:":
+                    raise RuntimeError(f"{src}: kernel {name} has {key} {value}; its inline-assembly schedule "
+                                       "needs every operand and accumulator in registers")
+    return checked
+
+
 def _compile(src, force):
     obj = os.path.join(OBJ, src.replace("/", "_") + ".o")
     path = os.path.join(CSRC, src)
     if force or _stale(obj, [path] + _headers()):
         flags = CXXFLAGS + (DEVICE_FLAGS if src.endswith(".hip") else [])
-        if src.startswith("driver/"):
+        if src.startswith("driver/") or src.startswith("probe/"):
             flags = flags + ["-fopenmp"]
-        _run([HIPCC] + flags + ["-c", path, "-o", obj])
+        if src.endswith(".hip"):
+            flags = flags + ["-Rpass-analysis=kernel-resource-usage"]
+        out = _run([HIPCC] + flags + ["-c", path, "-o", obj])
+        if src.endswith(".hip"):
+            try:
+                _check_no_spills(src, out)
+            except RuntimeError:
+                os.remove(obj)
+                raise
     return obj
 
 
 def build(force: bool = False, verbose: bool = False) -> dict:
     for d in (OBJ, LIB, BIN):
         os.makedirs(d, exist_ok=True)
-    sources = LIB_SOURCES + VENDOR_SOURCES + DRIVER_SOURCES
+    sources = LIB_SOURCES + VENDOR_SOURCES + DRIVER_SOURCES + PROBE_SOURCES
     with cf.ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
         objs = dict(zip(sources, pool.map(lambda s: _compile(s, force), sources)))
     libhgemm = os.path.join(LIB, "libhgemm.so")
@@ -87,9 +122,13 @@ def build(force: bool = False, verbose: bool = False) -> dict:
     if force or _stale(driver, drv_objs + [libhgemm, vendor]):
         _run([HIPCC, "-o", driver] + drv_objs + ["-L" + LIB, "-lhgemm", "-lhgemm_hipblaslt", "-fopenmp",
                                                   "-Wl,-rpath,$ORIGIN/../lib"])
+    probe = os.path.join(BIN, "hgemm_probe")
+    probe_objs = [objs[s] for s in PROBE_SOURCES]
+    if force or _stale(probe, probe_objs):
+        _run([HIPCC, "-o", probe] + probe_objs + ["-fopenmp"])
     if verbose:
-        print("built", libhgemm, vendor, driver)
-    return {"libhgemm": libhgemm, "vendor": vendor, "driver": driver}
+        print("built", libhgemm, vendor, driver, probe)
+    return {"libhgemm": libhgemm, "vendor": vendor, "driver": driver, "probe": probe}
 
 
 if __name__ == "__main__":

@@ -12,6 +12,11 @@ HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_pg2s_ps2r);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_stage2);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_stage3);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_stage4);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_64x64);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_128x128);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_192x192);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_256x128);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_256x256);
 HGEMM_DECLARE_SUPPORTS(hgemm_skinny);
 HGEMM_DECLARE_SUPPORTS(hgemm_auto);
 
@@ -43,6 +48,18 @@ const Variant kVariants[] = {
     {"Mfma-Async-Stage2", "hgemm_mfma_async_stage2", hgemm_mfma_async_stage2, hgemm_mfma_async_stage2_supports, 1},
     {"Mfma-Async-Stage3", "hgemm_mfma_async_stage3", hgemm_mfma_async_stage3, hgemm_mfma_async_stage3_supports, 1},
     {"Mfma-Async-Stage4", "hgemm_mfma_async_stage4", hgemm_mfma_async_stage4, hgemm_mfma_async_stage4_supports, 1},
+    // the tuned kernel, one entry per tile, smallest first: the ladder ends at its fastest rung,
+    // as the reference's run ends at mmaAsyncStage4 (src/main.cu:123)
+    {"Mfma-Pipelined-64x64", "hgemm_mfma_pipelined_64x64", hgemm_mfma_pipelined_64x64,
+     hgemm_mfma_pipelined_64x64_supports, 1},
+    {"Mfma-Pipelined-128x128", "hgemm_mfma_pipelined_128x128", hgemm_mfma_pipelined_128x128,
+     hgemm_mfma_pipelined_128x128_supports, 1},
+    {"Mfma-Pipelined-192x192", "hgemm_mfma_pipelined_192x192", hgemm_mfma_pipelined_192x192,
+     hgemm_mfma_pipelined_192x192_supports, 1},
+    {"Mfma-Pipelined-256x128", "hgemm_mfma_pipelined_256x128", hgemm_mfma_pipelined_256x128,
+     hgemm_mfma_pipelined_256x128_supports, 1},
+    {"Mfma-Pipelined-256x256", "hgemm_mfma_pipelined_256x256", hgemm_mfma_pipelined_256x256,
+     hgemm_mfma_pipelined_256x256_supports, 1},
     {"Skinny", "hgemm_skinny", hgemm_skinny, hgemm_skinny_supports, 1},
     {"Auto", "hgemm_auto", hgemm_auto, hgemm_auto_supports, 1},
 };

@@ -11,9 +11,10 @@ namespace hgemm {
 // uses && and lets edge threads run out of bounds, src/simt_naive.cu:14).
 __global__ void __launch_bounds__(256)
     simt_naive_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C, size_t M,
-                      size_t N, size_t K) {
-    const size_t row = threadIdx.y + (size_t)blockDim.y * blockIdx.y;
-    const size_t col = threadIdx.x + (size_t)blockDim.x * blockIdx.x;
+                      size_t N, size_t K, unsigned blocks_n) {
+    // one-dimensional grid (row-major over 16x16 blocks of C): no 65535 limit on either dimension
+    const size_t row = threadIdx.y + (size_t)blockDim.y * (blockIdx.x / blocks_n);
+    const size_t col = threadIdx.x + (size_t)blockDim.x * (blockIdx.x % blocks_n);
     if (row >= M || col >= N) return;
     float tmp = 0.0f;
     for (size_t i = 0; i < K; ++i) tmp += (float)A[row * K + i] * (float)B[i + col * K];
@@ -28,7 +29,8 @@ __global__ void __launch_bounds__(64)
     mfma_naive_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C, int N,
                       int K) {
     const int lane = threadIdx.x;
-    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int tiles_n = N / 32;  // one-dimensional grid, row-major over the 32x32 tiles of C
+    const int m0 = (int)(blockIdx.x / tiles_n) * 32, n0 = (int)(blockIdx.x % tiles_n) * 32;
     const half_t *a = A + (size_t)(m0 + (lane & 31)) * K + (lane >> 5) * 8;
     const half_t *b = B + (size_t)(n0 + (lane & 31)) * K + (lane >> 5) * 8;
     floatx16 acc;
@@ -57,10 +59,11 @@ extern "C" void hgemm_simt_naive(const hgemm_half *A, const hgemm_half *B, hgemm
                                  size_t K) {
     check_operands(A, B, C, M, N, K);
     dim3 block(16, 16);
-    dim3 grid((unsigned)div_ceil(N, block.x), (unsigned)div_ceil(M, block.y));
+    const unsigned blocks_n = (unsigned)div_ceil(N, block.x);
+    dim3 grid(blocks_n * (unsigned)div_ceil(M, block.y));
     simt_naive_kernel<<<grid, block, 0, nullptr>>>(reinterpret_cast<const half_t *>(A),
                                                    reinterpret_cast<const half_t *>(B),
-                                                   reinterpret_cast<half_t *>(C), M, N, K);
+                                                   reinterpret_cast<half_t *>(C), M, N, K, blocks_n);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 
@@ -69,7 +72,7 @@ extern "C" void hgemm_mfma_naive(const hgemm_half *A, const hgemm_half *B, hgemm
     check_operands(A, B, C, M, N, K);
     HGEMM_CHECK_MSG(M % 32 == 0 && N % 32 == 0 && K % 16 == 0,
                     "hgemm_mfma_naive needs M %% 32 == 0, N %% 32 == 0, K %% 16 == 0 (got M=%zu N=%zu K=%zu)", M, N, K);
-    dim3 grid((unsigned)(N / 32), (unsigned)(M / 32));
+    dim3 grid((unsigned)((N / 32) * (M / 32)));
     mfma_naive_kernel<<<grid, dim3(64), 0, nullptr>>>(reinterpret_cast<const half_t *>(A),
                                                       reinterpret_cast<const half_t *>(B),
                                                       reinterpret_cast<half_t *>(C), (int)N, (int)K);

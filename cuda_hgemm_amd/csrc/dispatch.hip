@@ -6,40 +6,64 @@
 #include "mfma_skinny.h"
 #include "plan.h"
 
+#include <mutex>
+
 namespace hgemm {
 
 namespace {
 
-// Process-lifetime fp32 workspace for split-K partial sums; grows on demand, never freed
-// (the reference keeps its vendor handle the same way, src/cublas_tensor_op.cu:18).
-float *splitk_workspace(size_t bytes) {
-    static float *ptr = nullptr;
-    static size_t capacity = 0;
-    if (bytes > capacity) {
-        if (ptr) {
-            HGEMM_CHECK_HIP_ERROR(hipDeviceSynchronize());  // earlier launches may still use it
-            HGEMM_CHECK_HIP_ERROR(hipFree(ptr));
-        }
-        size_t want = bytes < (64ull << 20) ? (64ull << 20) : bytes;
-        HGEMM_CHECK_HIP_ERROR(hipMalloc(reinterpret_cast<void **>(&ptr), want));
-        capacity = want;
-    }
-    return ptr;
+constexpr size_t MAX_PARTIAL_BYTES = PlanLimits().partial_bytes;
+constexpr size_t MAX_PADDED_BYTES = PlanLimits().operand_bytes;
+constexpr int MAX_DEVICES = 64;
+
+int current_device() {
+    int dev = 0;
+    HGEMM_CHECK_HIP_ERROR(hipGetDevice(&dev));
+    HGEMM_CHECK_MSG(dev >= 0 && dev < MAX_DEVICES, "device %d beyond the %d this library keeps state for", dev, MAX_DEVICES);
+    return dev;
 }
 
-// Same, for zero-padded copies of the operands of shapes whose rows are not aligned.
-unsigned char *operand_workspace(size_t bytes) {
-    static unsigned char *ptr = nullptr;
-    static size_t capacity = 0;
-    if (bytes > capacity) {
-        if (ptr) {
-            HGEMM_CHECK_HIP_ERROR(hipDeviceSynchronize());
-            HGEMM_CHECK_HIP_ERROR(hipFree(ptr));
-        }
-        HGEMM_CHECK_HIP_ERROR(hipMalloc(reinterpret_cast<void **>(&ptr), bytes));
-        capacity = bytes;
+// Heap workspaces of hgemm_auto / hgemm_skinny, one pair per device, kept for the life of
+// the process (the reference keeps its vendor handle the same way,
+// src/cublas_tensor_op.cu:18).  Each is allocated once, at its cap, the first time a plan
+// needs it (or by hgemm_reserve_workspace), so a later call with a larger shape never
+// reallocates: no hipFree, no device synchronisation inside an entry point.  If the cap
+// cannot be had, the size asked for is tried; if that fails too the caller plans again
+// without a workspace.
+std::mutex g_heap_mutex;
+Workspace g_heap[MAX_DEVICES];
+
+bool grow(void **ptr, size_t *have, size_t need, size_t cap) {
+    if (need <= *have) return true;
+    if (*ptr) {  // only hgemm_reserve_workspace can ask for more than the cap that was allocated
+        HGEMM_CHECK_HIP_ERROR(hipDeviceSynchronize());
+        HGEMM_CHECK_HIP_ERROR(hipFree(*ptr));
+        *ptr = nullptr;
+        *have = 0;
     }
-    return ptr;
+    for (size_t want : {need > cap ? need : cap, need}) {
+        if (hipMalloc(ptr, want) == hipSuccess) {
+            *have = want;
+            return true;
+        }
+        (void)hipGetLastError();  // clear the allocation failure
+        *ptr = nullptr;
+    }
+    return false;
+}
+
+// The device's heap workspace with at least the given sizes; false if memory ran out.
+bool heap_workspace(size_t partial_bytes, size_t operand_bytes, Workspace *out) {
+    const int dev = current_device();
+    std::lock_guard<std::mutex> lock(g_heap_mutex);
+    Workspace &w = g_heap[dev];
+    bool ok = true;
+    if (partial_bytes > w.partial_bytes)
+        ok = grow(reinterpret_cast<void **>(&w.partial), &w.partial_bytes, partial_bytes, MAX_PARTIAL_BYTES) && ok;
+    if (operand_bytes > w.operand_bytes)
+        ok = grow(reinterpret_cast<void **>(&w.operands), &w.operand_bytes, operand_bytes, MAX_PADDED_BYTES) && ok;
+    *out = w;
+    return ok;
 }
 
 int compute_units() {
@@ -54,7 +78,8 @@ int compute_units() {
 }
 
 template <class Cfg>
-void launch_splitk(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, int splits) {
+void launch_splitk(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, int splits,
+                   const Workspace &ws) {
     static bool configured = [] {
         HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_skinny_kernel<Cfg>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
@@ -63,11 +88,17 @@ void launch_splitk(const void *A, const void *B, void *C, size_t M, size_t N, si
     (void)configured;
     HGEMM_CHECK(N % Cfg::BN == 0);
     HGEMM_CHECK(splits >= 1 && K % ((size_t)splits * Cfg::BK) == 0);
-    const dim3 grid((unsigned)(N / Cfg::BN), (unsigned)div_ceil(M, Cfg::BM), (unsigned)splits);
-    float *partial = splits > 1 ? splitk_workspace((size_t)splits * M * N * sizeof(float)) : nullptr;
+    const size_t tiles_n = N / Cfg::BN, tiles = tiles_n * div_ceil(M, Cfg::BM);  // < 2^31 / (BM * BN)
+    const dim3 grid((unsigned)tiles, (unsigned)splits);
+    HGEMM_CHECK(splits <= 65535);
+    float *partial = nullptr;
+    if (splits > 1) {
+        HGEMM_CHECK(ws.partial != nullptr && ws.partial_bytes >= (size_t)splits * M * N * sizeof(float));
+        partial = ws.partial;
+    }
     hgemm_skinny_kernel<Cfg><<<grid, dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
-        partial, (int)M, (int)N, (int)K, (int)(K / splits));
+        partial, (int)M, (int)N, (int)K, (int)(K / splits), (int)tiles_n);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
     if (splits > 1) launch_splitk_reduce(partial, reinterpret_cast<half_t *>(C), M * N, splits);
 }
@@ -91,7 +122,8 @@ using Rect256x128 = PipeConfig<256, 128, 64, 2, 2, 3, 16>;
 // ordered reduction (the same one the small-M kernel uses), so the result is bit-identical
 // from run to run.
 template <class Cfg>
-void launch_pipelined_plan(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, const Plan &plan) {
+void launch_pipelined_plan(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, const Plan &plan,
+                           const Workspace &ws) {
     const int splits = plan.splits;
     if constexpr (Cfg::BM == 256 && Cfg::BN == 256) {
         switch (plan.tail_kernel) {
@@ -108,17 +140,18 @@ void launch_pipelined_plan(const void *A, const void *B, void *C, size_t M, size
         }
     }
     if (plan.tail_splits > 1) {
-        float *partial = splitk_workspace((size_t)plan.tail_splits * plan.tail_tiles * Cfg::BM * Cfg::BN * sizeof(float));
-        launch_pipelined_with_tail<Cfg>(A, B, C, partial, M, N, K, plan.tail_tiles, plan.tail_splits, "hgemm_auto");
+        HGEMM_CHECK(ws.partial != nullptr &&
+                    ws.partial_bytes >= (size_t)plan.tail_splits * plan.tail_tiles * Cfg::BM * Cfg::BN * sizeof(float));
+        launch_pipelined_with_tail<Cfg>(A, B, C, ws.partial, M, N, K, plan.tail_tiles, plan.tail_splits, "hgemm_auto");
         return;
     }
     if (splits <= 1) {
         launch_pipelined<Cfg>(A, B, C, M, N, K, "hgemm_auto");
         return;
     }
-    float *partial = splitk_workspace((size_t)splits * M * N * sizeof(float));
-    launch_pipelined_split<Cfg>(A, B, partial, M, N, K, splits, "hgemm_auto");
-    launch_splitk_reduce(partial, reinterpret_cast<half_t *>(C), M * N, splits);
+    HGEMM_CHECK(ws.partial != nullptr && ws.partial_bytes >= (size_t)splits * M * N * sizeof(float));
+    launch_pipelined_split<Cfg>(A, B, ws.partial, M, N, K, splits, "hgemm_auto");
+    launch_splitk_reduce(ws.partial, reinterpret_cast<half_t *>(C), M * N, splits);
 }
 
 // ---- cost model for the tile-aligned shapes.  A candidate is a tile (its kernel), how
@@ -144,8 +177,6 @@ constexpr Candidate CANDIDATES[] = {
 constexpr double LAUNCH_US = 0.16, REDUCE_US = 3.90, REDUCE_SLICE_US = 0.10, REDUCE_BYTES_PER_US = 7040e3;
 // extra cost of finishing a grid with a separate launch for its last round: in K slices / on smaller tiles
 constexpr double TAIL_US = 3.6, TAIL_SUB_US = 4.4;
-constexpr size_t MAX_PARTIAL_BYTES = 512ull << 20;
-constexpr size_t MAX_PADDED_BYTES = 1024ull << 20;
 size_t padded_n(size_t N) { return (N + 7) / 8 * 8; }
 size_t padded_k(size_t K) { return (K + 63) / 64 * 64; }
 // A' (M x K'), B' (N' x K') and, when N grows, C' (M x N')
@@ -199,9 +230,12 @@ double predict_subtile_us(const Candidate &big, const Candidate &small, size_t M
 // gives at least three quarters of the CUs a workgroup.  Each slice is a whole number of 64-wide chunks, at least
 // two of them.  (Measured on the decode shapes: more slices than that only add partial-sum
 // traffic, fewer leave CUs without a stream of B.)
-int choose_splits(size_t tiles, size_t cus, size_t K) {
+// `slice_bytes`: fp32 partial sums of one slice; the slices together stay within `limit`.
+int choose_splits(size_t tiles, size_t cus, size_t K, size_t slice_bytes, size_t limit) {
     int s = 1;
-    while (s < 16 && tiles * s < cus * 3 / 4 && K % ((size_t)s * 2 * 64) == 0 && K / (s * 2) >= 128) s *= 2;
+    while (s < 16 && tiles * s < cus * 3 / 4 && K % ((size_t)s * 2 * 64) == 0 && K / (s * 2) >= 128 &&
+           (size_t)(s * 2) * slice_bytes <= limit)
+        s *= 2;
     return s;
 }
 
@@ -214,10 +248,11 @@ bool skinny_supports(size_t M, size_t N, size_t K) {
 // M <= 128: choices come from timing every candidate (tile x slices) on the specification's
 // decode shapes on an MI355X, operands rotated so small problems read HBM.  Larger,
 // tile-aligned shapes: the cheapest (tile, slices) pair under the cost model above.
-Plan plan_for(size_t M, size_t N, size_t K) {
+Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     Plan p;
     if (M == 0 || N == 0 || K == 0) return p;
     const size_t cus = (size_t)compute_units();
+    const size_t slice_bytes = M * N * sizeof(float);  // fp32 partial sums of one K slice of the whole product
     if (M <= 8 && decode_supports(M, N, K)) {  // a few rows: one streaming pass over B, no second launch
         int bn = 16, waves = 1;
         decode_plan(M, N, K, cus, &bn, &waves);
@@ -237,7 +272,8 @@ Plan plan_for(size_t M, size_t N, size_t K) {
             p.kernel = wide ? KERNEL_SPLIT_64x128 : KERNEL_SPLIT_64x64;
         else
             p.kernel = wide ? KERNEL_SPLIT_128x128 : KERNEL_SPLIT_128x64;
-        p.splits = choose_splits(N / (wide ? 128 : 64), cus, K);
+        p.splits = choose_splits(N / (wide ? 128 : 64), cus, K, slice_bytes, limits.partial_bytes);
+        if (p.splits > 1) p.partial_bytes = (size_t)p.splits * slice_bytes;
         return p;
     }
     // Pipelined tiles: M and N may end inside a tile (guarded edges; the model charges whole
@@ -247,7 +283,7 @@ Plan plan_for(size_t M, size_t N, size_t K) {
         if (N % 8) break;
         for (int s = 1; s <= 32; s *= 2) {
             if (K % ((size_t)s * 64) || K / s < (size_t)64 * c.stages) break;
-            if (s > 1 && (size_t)s * M * N * sizeof(float) > MAX_PARTIAL_BYTES) break;
+            if (s > 1 && (size_t)s * slice_bytes > limits.partial_bytes) break;
             const double t = predict_us(c, M, N, K, s, cus);
             if (p.kernel == KERNEL_NONE || t < best) {
                 best = t;
@@ -257,6 +293,7 @@ Plan plan_for(size_t M, size_t N, size_t K) {
                 p.tail_tiles = 0;
                 p.tail_splits = 1;
                 p.tail_kernel = KERNEL_NONE;
+                p.partial_bytes = s > 1 ? (size_t)s * slice_bytes : 0;
             }
         }
         // a grid of whole rounds plus a few workgroups: run those few in K slices
@@ -265,7 +302,7 @@ Plan plan_for(size_t M, size_t N, size_t K) {
         if (wgs > slots && rem > 0) {
             for (int ts = 2; ts <= 16; ts *= 2) {
                 if (K % ((size_t)ts * 64) || K / ts < (size_t)64 * c.stages || rem * ts > slots) break;
-                if ((size_t)ts * rem * c.bm * c.bn * sizeof(float) > MAX_PARTIAL_BYTES) break;
+                if ((size_t)ts * rem * c.bm * c.bn * sizeof(float) > limits.partial_bytes) break;
                 const double t = predict_tail_us(c, M, N, K, ts, cus);
                 if (p.kernel != KERNEL_NONE && t < best) {
                     best = t;
@@ -275,6 +312,7 @@ Plan plan_for(size_t M, size_t N, size_t K) {
                     p.tail_tiles = (int)rem;
                     p.tail_splits = ts;
                     p.tail_kernel = KERNEL_NONE;
+                    p.partial_bytes = (size_t)ts * rem * c.bm * c.bn * sizeof(float);
                 }
             }
             if (c.kernel == KERNEL_BIG256) {  // ... or on smaller tiles that divide this one
@@ -290,6 +328,7 @@ Plan plan_for(size_t M, size_t N, size_t K) {
                         p.tail_tiles = (int)rem;
                         p.tail_splits = 1;
                         p.tail_kernel = small.kernel;
+                        p.partial_bytes = 0;
                     }
                 }
             }
@@ -298,7 +337,8 @@ Plan plan_for(size_t M, size_t N, size_t K) {
     if (p.kernel != KERNEL_NONE) return p;
     if (N % 64 == 0 && K % 64 == 0) {  // any M: rows beyond M are guarded
         p.kernel = KERNEL_SPLIT_64x64;
-        p.splits = choose_splits(div_ceil(M, 64) * (N / 64), cus, K);
+        p.splits = choose_splits(div_ceil(M, 64) * (N / 64), cus, K, slice_bytes, limits.partial_bytes);
+        if (p.splits > 1) p.partial_bytes = (size_t)p.splits * slice_bytes;
         return p;
     }
     // Rows of C not 16-byte aligned (N % 8) or K not a whole number of chunks.  Large
@@ -306,8 +346,8 @@ Plan plan_for(size_t M, size_t N, size_t K) {
     // shape the pipelined kernels take and run that (same products, same result); the rest
     // goes to the guarded kernel, which sustains about 80 TFLOP/s.
     const size_t Np = padded_n(N), Kp = padded_k(K);
-    if (K >= 192 && padded_bytes(M, N, K) <= MAX_PADDED_BYTES) {
-        const Plan inner = plan_for(M, Np, Kp);
+    if (K >= 192 && padded_bytes(M, N, K) <= limits.operand_bytes) {
+        const Plan inner = plan_for(M, Np, Kp, limits);
         const double inner_us = inner.est_us > 0.0 ? inner.est_us : 8.0 + (double)(Np * Kp * 2) / 4e6;
         const double copy_us = 6.0 + 4.0 * (double)((M + Np) * Kp + (Np != N ? M * Np : 0)) / 3.5e6;
         const double guarded_us = 5.0 + 2.0 * (double)M * (double)N * (double)K / 80e6;
@@ -315,6 +355,8 @@ Plan plan_for(size_t M, size_t N, size_t K) {
             p.kernel = KERNEL_PADDED;
             p.splits = inner.splits;
             p.est_us = copy_us + inner_us;
+            p.partial_bytes = inner.partial_bytes;
+            p.operand_bytes = padded_bytes(M, N, K);
             return p;
         }
     }
@@ -356,19 +398,25 @@ __global__ void __launch_bounds__(256)
     dst[i] = src[r * cols_src + c];
 }
 
-void run_padded(const void *A, const void *B, void *C, size_t M, size_t N, size_t K) {
+void run_padded(const Plan &p, const Workspace &ws, const void *A, const void *B, void *C, size_t M, size_t N,
+                size_t K) {
     const size_t Np = padded_n(N), Kp = padded_k(K);
-    unsigned char *ws = operand_workspace(padded_bytes(M, N, K));
-    half_t *Ap = reinterpret_cast<half_t *>(ws), *Bp = Ap + M * Kp;
+    HGEMM_CHECK(ws.operands != nullptr && ws.operand_bytes >= padded_bytes(M, N, K));
+    half_t *Ap = reinterpret_cast<half_t *>(ws.operands), *Bp = Ap + M * Kp;
     half_t *Cp = Np != N ? Bp + Np * Kp : reinterpret_cast<half_t *>(C);
     pad_copy_kernel<<<dim3((unsigned)div_ceil(M * (Kp / 8), (size_t)256)), dim3(256), 0, nullptr>>>(
         reinterpret_cast<const half_t *>(A), Ap, (int)M, (int)K, (int)M, (int)Kp);
     pad_copy_kernel<<<dim3((unsigned)div_ceil(Np * (Kp / 8), (size_t)256)), dim3(256), 0, nullptr>>>(
         reinterpret_cast<const half_t *>(B), Bp, (int)N, (int)K, (int)Np, (int)Kp);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
-    const Plan inner = plan_for(M, Np, Kp);
-    HGEMM_CHECK(inner.kernel != KERNEL_PADDED && inner.kernel != KERNEL_RAGGED);
-    run_plan(inner, Ap, Bp, Cp, M, Np, Kp);
+    // The inner plan that plan_for sized p for: the best plan within a limit is still the best
+    // within the smaller limit of what it needs itself.
+    PlanLimits inner_limits;
+    inner_limits.partial_bytes = p.partial_bytes;
+    inner_limits.operand_bytes = 0;
+    const Plan inner = plan_for(M, Np, Kp, inner_limits);
+    HGEMM_CHECK(inner.kernel != KERNEL_PADDED && inner.kernel != KERNEL_RAGGED && inner.partial_bytes == p.partial_bytes);
+    run_plan(inner, ws, Ap, Bp, Cp, M, Np, Kp);
     if (Np != N) {
         unpad_copy_kernel<<<dim3((unsigned)div_ceil(M * N, (size_t)256)), dim3(256), 0, nullptr>>>(
             Cp, reinterpret_cast<half_t *>(C), (int)M, (int)Np, (int)N);
@@ -376,23 +424,24 @@ void run_padded(const void *A, const void *B, void *C, size_t M, size_t N, size_
     }
 }
 
-void run_plan(const Plan &p, const void *A, const void *B, void *C, size_t M, size_t N, size_t K) {
+void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, void *C, size_t M, size_t N,
+              size_t K) {
     switch (p.kernel) {
-        case KERNEL_BIG256: launch_pipelined_plan<Big256>(A, B, C, M, N, K, p); break;
-        case KERNEL_T192: launch_pipelined_plan<Tile192>(A, B, C, M, N, K, p); break;
-        case KERNEL_R256x128: launch_pipelined_plan<Rect256x128>(A, B, C, M, N, K, p); break;
-        case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p); break;
+        case KERNEL_BIG256: launch_pipelined_plan<Big256>(A, B, C, M, N, K, p, ws); break;
+        case KERNEL_T192: launch_pipelined_plan<Tile192>(A, B, C, M, N, K, p, ws); break;
+        case KERNEL_R256x128: launch_pipelined_plan<Rect256x128>(A, B, C, M, N, K, p, ws); break;
+        case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128_S4: launch_pipelined<Mid128S4>(A, B, C, M, N, K, "hgemm_auto"); break;
-        case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p); break;
-        case KERNEL_SPLIT_32x64: launch_splitk<Split32x64>(A, B, C, M, N, K, p.splits); break;
-        case KERNEL_SPLIT_64x64: launch_splitk<Split64x64>(A, B, C, M, N, K, p.splits); break;
-        case KERNEL_SPLIT_64x128: launch_splitk<Split64x128>(A, B, C, M, N, K, p.splits); break;
-        case KERNEL_SPLIT_128x64: launch_splitk<Split128x64>(A, B, C, M, N, K, p.splits); break;
-        case KERNEL_SPLIT_128x128: launch_splitk<Split128x128>(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p, ws); break;
+        case KERNEL_SPLIT_32x64: launch_splitk<Split32x64>(A, B, C, M, N, K, p.splits, ws); break;
+        case KERNEL_SPLIT_64x64: launch_splitk<Split64x64>(A, B, C, M, N, K, p.splits, ws); break;
+        case KERNEL_SPLIT_64x128: launch_splitk<Split64x128>(A, B, C, M, N, K, p.splits, ws); break;
+        case KERNEL_SPLIT_128x64: launch_splitk<Split128x64>(A, B, C, M, N, K, p.splits, ws); break;
+        case KERNEL_SPLIT_128x128: launch_splitk<Split128x128>(A, B, C, M, N, K, p.splits, ws); break;
         case KERNEL_DECODE_BN16: launch_decode(A, B, C, M, N, K, 16, p.splits); break;
         case KERNEL_DECODE_BN32: launch_decode(A, B, C, M, N, K, 32, p.splits); break;
         case KERNEL_RAGGED: launch_ragged(A, B, C, M, N, K); break;
-        case KERNEL_PADDED: run_padded(A, B, C, M, N, K); break;
+        case KERNEL_PADDED: run_padded(p, ws, A, B, C, M, N, K); break;
         case KERNEL_SIMT:
             hgemm_simt_naive(reinterpret_cast<const hgemm_half *>(A), reinterpret_cast<const hgemm_half *>(B),
                              reinterpret_cast<hgemm_half *>(C), M, N, K);
@@ -405,17 +454,94 @@ void run_plan(const Plan &p, const void *A, const void *B, void *C, size_t M, si
 
 using namespace hgemm;
 
+namespace {
+
+// Plans of the shapes this thread saw last: a 5 us launch should not re-run the cost model
+// (five tiles x K slices x tails, in doubles) on every call.  Direct-mapped, fixed size,
+// per thread: no allocation, no lock.
+struct CachedPlan {
+    size_t M = 0, N = 0, K = 0;
+    Plan plan;
+};
+constexpr int PLAN_CACHE_SLOTS = 64;
+
+const Plan &cached_plan(size_t M, size_t N, size_t K) {
+    static thread_local CachedPlan cache[PLAN_CACHE_SLOTS];
+    const size_t h = (M * 0x9e3779b97f4a7c15ull) ^ (N * 0xc2b2ae3d27d4eb4full) ^ (K * 0x165667b19e3779f9ull);
+    CachedPlan &slot = cache[(h >> 32) % PLAN_CACHE_SLOTS];
+    if (slot.M != M || slot.N != N || slot.K != K) {
+        slot.plan = plan_for(M, N, K);
+        slot.M = M, slot.N = N, slot.K = K;
+    }
+    return slot.plan;
+}
+
+// Runs the cached plan of the shape on the heap workspace; when device memory for the
+// workspace cannot be had, the best plan that needs none (no K slices, the guarded kernel
+// instead of padded copies).
+void run_with_heap_workspace(const void *A, const void *B, void *C, size_t M, size_t N, size_t K) {
+    const Plan &p = cached_plan(M, N, K);
+    Workspace ws;
+    if (p.partial_bytes == 0 && p.operand_bytes == 0) {
+        run_plan(p, ws, A, B, C, M, N, K);
+    } else if (heap_workspace(p.partial_bytes, p.operand_bytes, &ws)) {
+        run_plan(p, ws, A, B, C, M, N, K);
+    } else {
+        PlanLimits none;
+        none.partial_bytes = none.operand_bytes = 0;
+        run_plan(plan_for(M, N, K, none), Workspace(), A, B, C, M, N, K);
+    }
+}
+
+}  // namespace
+
 extern "C" void hgemm_skinny(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K) {
     check_operands(A, B, C, M, N, K);
     HGEMM_CHECK_MSG(skinny_supports(M, N, K),
                     "hgemm_skinny needs M <= 128, N %% 64 == 0, K %% 64 == 0 (got M=%zu N=%zu K=%zu)", M, N, K);
-    run_plan(plan_for(M, N, K), A, B, C, M, N, K);
+    run_with_heap_workspace(A, B, C, M, N, K);
 }
 extern "C" int hgemm_skinny_supports(size_t M, size_t N, size_t K) { return skinny_supports(M, N, K) ? 1 : 0; }
 
 extern "C" void hgemm_auto(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K) {
     check_operands(A, B, C, M, N, K);
-    run_plan(plan_for(M, N, K), A, B, C, M, N, K);
+    run_with_heap_workspace(A, B, C, M, N, K);
+}
+
+// The tuned kernel by tile, as entry points of their own.  M and N may end inside a tile.
+#define HGEMM_DEFINE_PIPELINED_VARIANT(symbol, Cfg)                                                          \
+    extern "C" void symbol(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N,      \
+                           size_t K) {                                                                       \
+        launch_pipelined<Cfg>(A, B, C, M, N, K, #symbol);                                                    \
+    }                                                                                                        \
+    extern "C" int symbol##_supports(size_t M, size_t N, size_t K) {                                         \
+        return pipelined_supports_edges<Cfg>(M, N, K) ? 1 : 0;                                               \
+    }
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_64x64, Small64)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_128x128, Mid128)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_192x192, Tile192)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_256x128, Rect256x128)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_256x256, Big256)
+
+extern "C" int hgemm_reserve_workspace(size_t partial_bytes, size_t operand_bytes) {
+    Workspace ws;
+    return heap_workspace(partial_bytes, operand_bytes, &ws) ? 0 : 1;
+}
+
+extern "C" void hgemm_release_workspace(void) {
+    const int dev = current_device();
+    std::lock_guard<std::mutex> lock(g_heap_mutex);
+    Workspace &w = g_heap[dev];
+    if (w.partial || w.operands) HGEMM_CHECK_HIP_ERROR(hipDeviceSynchronize());  // launches may still use them
+    if (w.partial) HGEMM_CHECK_HIP_ERROR(hipFree(w.partial));
+    if (w.operands) HGEMM_CHECK_HIP_ERROR(hipFree(w.operands));
+    w = Workspace();
+}
+
+extern "C" size_t hgemm_auto_workspace_bytes(size_t M, size_t N, size_t K, size_t *operand_bytes) {
+    const Plan p = plan_for(M, N, K);
+    if (operand_bytes) *operand_bytes = p.operand_bytes;
+    return p.partial_bytes;
 }
 extern "C" int hgemm_auto_supports(size_t M, size_t N, size_t K) { return M > 0 && N > 0 && K > 0; }
 

@@ -11,12 +11,14 @@
 
 using namespace hgemm;
 
-static void write_json(const std::string &path, const Tester &tester, size_t M, size_t N, size_t K,
+static void write_json(const std::string &path, const Tester &tester, size_t M, size_t N, size_t K, uint64_t seed,
                        const hipDeviceProp_t &prop) {
     FILE *f = fopen(path.c_str(), "w");
     HGEMM_CHECK_MSG(f != nullptr, "cannot write %s", path.c_str());
     fprintf(f, "{\"device\": \"%s\", \"compute_units\": %d, \"clock_mhz\": %.0f, \"M\": %zu, \"N\": %zu, \"K\": %zu,\n",
             prop.name, prop.multiProcessorCount, prop.clockRate * 1e-3, M, N, K);
+    fprintf(f, " \"seed\": %llu, \"a_checksum\": \"0x%016llx\", \"b_checksum\": \"0x%016llx\",\n",
+            (unsigned long long)seed, (unsigned long long)tester.checksumA(), (unsigned long long)tester.checksumB());
     fprintf(f, " \"flops\": %.6e, \"bytes\": %.6e, \"results\": [\n", 2.0 * M * N * K, hgemm_bytes(M, N, K));
     const auto &recs = tester.records();
     for (size_t i = 0; i < recs.size(); ++i) {
@@ -51,7 +53,7 @@ int main(int argc, char *argv[]) {
     flags.define("dist_b", "uniform", "distribution of B");
     flags.define("rotate_mb", "0", "cycle over operand sets totalling at least this many MB (HBM-cold timing)");
     flags.define("json", "", "also write the results to this file as JSON");
-    flags.define("probe", "0", "launches of the in-kernel timing probe of the tuned kernel (0: off; needs M, N % 256 == 0)");
+    flags.define("fill_only", "false", "generate A and B on the host, print their checksums and exit (no GPU needed)");
     flags.parse(argc, argv);
 
     const size_t M = flags.u64("M"), N = flags.u64("N"), K = flags.u64("K");
@@ -60,6 +62,15 @@ int main(int argc, char *argv[]) {
     HGEMM_CHECK_GT(cpu_procs, 0);
 
     omp_set_num_threads(cpu_procs);
+    if (flags.boolean("fill_only")) {
+        std::vector<_Float16> a(M * K), b(K * N);
+        fill_host(a.data(), a.size(), flags.u64("seed"), 1, parse_fill(flags.str("dist_a")));
+        fill_host(b.data(), b.size(), flags.u64("seed"), 2, parse_fill(flags.str("dist_b")));
+        printf("{\"M\": %zu, \"N\": %zu, \"K\": %zu, \"seed\": %zu, \"a_checksum\": \"0x%016llx\", \"b_checksum\": \"0x%016llx\"}\n",
+               M, N, K, flags.u64("seed"), (unsigned long long)checksum64(a.data(), a.size()),
+               (unsigned long long)checksum64(b.data(), b.size()));
+        return 0;
+    }
     HGEMM_CHECK_HIP_ERROR(hipSetDevice(gpu_rank));
 
     hipDeviceProp_t prop;
@@ -118,9 +129,7 @@ int main(int argc, char *argv[]) {
         }
     }
 
-    if (flags.u64("probe") > 0) tester.probe(flags.u64("probe"));
-
-    if (!flags.str("json").empty()) write_json(flags.str("json"), tester, M, N, K, prop);
+    if (!flags.str("json").empty()) write_json(flags.str("json"), tester, M, N, K, flags.u64("seed"), prop);
 
     if (tester.failures() > 0) {
         HLOG("Done with %zu failed check(s)", tester.failures());

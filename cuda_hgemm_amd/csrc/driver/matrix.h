@@ -62,6 +62,41 @@ inline uint64_t mix64(uint64_t z) {
     return z ^ (z >> 31);
 }
 
+// Element i of matrix `stream` under `seed`: a counter-based generator, so a fill does not
+// depend on the thread count or on the order of evaluation.  Host code only.
+inline void fill_host(_Float16 *dst, size_t elems, uint64_t seed, uint64_t stream, const FillSpec &fill) {
+    const uint64_t key = mix64(seed ^ (stream * 0xd1342543de82ef95ull));
+    const long n = (long)elems;
+#pragma omp parallel for schedule(static)
+    for (long i = 0; i < n; ++i) {
+        const uint64_t r = mix64(key + (uint64_t)i * 0x9e3779b97f4a7c15ull);
+        float v = 0.0f;
+        if (fill.kind == Fill::Uniform) {
+            v = fill.p0 + (fill.p1 - fill.p0) * ((float)(r >> 40) * (1.0f / 16777216.0f));
+        } else if (fill.kind == Fill::Normal) {
+            const double u1 = ((double)(uint32_t)(r >> 32) + 1.0) * (1.0 / 4294967296.0);
+            const double u2 = (double)(uint32_t)r * (1.0 / 4294967296.0);
+            v = (float)(fill.p0 + fill.p1 * sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925 * u2));
+        }
+        dst[i] = (_Float16)v;  // round-to-nearest-even, as __float2half
+    }
+}
+
+// Position-dependent 64-bit checksum of fp16 bit patterns: sum of (bits + 1) * odd(i) mod
+// 2^64 with odd(i) = (i * 0x9e3779b97f4a7c15) | 1.  Goes into the JSON report so that a run's
+// inputs can be compared with another generator's for the same seed.
+inline uint64_t checksum64(const _Float16 *data, size_t elems) {
+    uint64_t sum = 0;
+    const long n = (long)elems;
+#pragma omp parallel for schedule(static) reduction(+ : sum)
+    for (long i = 0; i < n; ++i) {
+        uint16_t bits;
+        memcpy(&bits, &data[i], sizeof(bits));
+        sum += ((uint64_t)bits + 1u) * (((uint64_t)i * 0x9e3779b97f4a7c15ull) | 1u);
+    }
+    return sum;
+}
+
 class Matrix {
 public:
     Matrix(size_t row, size_t col, const std::string &name, uint64_t seed, uint64_t stream, const FillSpec &fill)
@@ -71,23 +106,8 @@ public:
         m_elem_num = m_row * m_col;
         m_host.resize(m_elem_num);
         HGEMM_CHECK_HIP_ERROR(hipMalloc(reinterpret_cast<void **>(&m_dev_ptr), m_elem_num * sizeof(_Float16)));
-
-        const uint64_t key = mix64(seed ^ (stream * 0xd1342543de82ef95ull));
-        _Float16 *dst = m_host.data();
-        const long n = (long)m_elem_num;
-#pragma omp parallel for schedule(static)
-        for (long i = 0; i < n; ++i) {
-            const uint64_t r = mix64(key + (uint64_t)i * 0x9e3779b97f4a7c15ull);
-            float v = 0.0f;
-            if (fill.kind == Fill::Uniform) {
-                v = fill.p0 + (fill.p1 - fill.p0) * ((float)(r >> 40) * (1.0f / 16777216.0f));
-            } else if (fill.kind == Fill::Normal) {
-                const double u1 = ((double)(uint32_t)(r >> 32) + 1.0) * (1.0 / 4294967296.0);
-                const double u2 = (double)(uint32_t)r * (1.0 / 4294967296.0);
-                v = (float)(fill.p0 + fill.p1 * sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925 * u2));
-            }
-            dst[i] = (_Float16)v;  // round-to-nearest-even, as __float2half
-        }
+        fill_host(m_host.data(), m_elem_num, seed, stream, fill);
+        m_fill_checksum = checksum64(m_host.data(), m_elem_num);
         moveToDevice();
         HLOG("%s: %zu * %zu, cpu: %p, gpu: %p", m_name.c_str(), m_row, m_col, (void *)m_host.data(), (void *)m_dev_ptr);
     }
@@ -152,6 +172,8 @@ public:
     double avgDiff() const { return m_avg_diff; }
     double baseRms() const { return m_base_rms; }
     size_t nonFinite() const { return m_non_finite; }
+    // checksum64 of the values the constructor generated (not of later host contents)
+    uint64_t fillChecksum() const { return m_fill_checksum; }
 
 private:
     const size_t m_row = 0;
@@ -162,6 +184,7 @@ private:
     uint16_t *m_dev_ptr = nullptr;
     double m_max_diff = 0.0, m_avg_diff = 0.0, m_base_rms = 0.0;
     size_t m_non_finite = 0;
+    uint64_t m_fill_checksum = 0;
 
     HGEMM_DISALLOW_COPY_AND_ASSIGN(Matrix);
 };

@@ -125,21 +125,9 @@ public:
         m_records.push_back(rec);
     }
 
-    // In-kernel timing of the tuned 256x256x64 kernel: the real kernel, its loop without
-    // copies, and without copies and operand reads (what the copies and the reads cost).
-    void probe(size_t launches) {
-        static const char *names[3] = {"tuned kernel", "loop without copies", "loop without copies and operand reads"};
-        for (int mode = 0; mode < 3; ++mode) {
-            double r[8];
-            hgemm_probe_loop(m_A->getDevPtr(), m_B->getDevPtr(), m_C->getDevPtr(), m_M, m_N, m_K, mode, launches, r);
-            HLOG("Probe %s: %zu launches avg %.4f ms, traced launch %.4f ms (%.1f TFLOPS); per workgroup: prologue "
-                 "%.2f us, loop %.2f us, epilogue %.2f us; loop %.0f shader cycles at %.3f GHz, MFMA issue %.1f%%",
-                 names[mode], launches, r[0], r[1], hgemm_tflops(m_M, m_N, m_K, r[1]), r[2], r[3], r[4], r[5], r[6],
-                 100.0 * r[7]);
-        }
-    }
-
     size_t failures() const { return m_failures; }
+    uint64_t checksumA() const { return m_A->fillChecksum(); }
+    uint64_t checksumB() const { return m_B->fillChecksum(); }
     const std::vector<EvalRecord> &records() const { return m_records; }
 
 private:

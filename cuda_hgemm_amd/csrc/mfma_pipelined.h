@@ -34,10 +34,12 @@ struct PipeConfig : TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_
     static constexpr int PKSTEP = MI == 32 ? 16 : 32;               // k covered by one MFMA
     static constexpr int PKSTEPS = BK_ / PKSTEP;
     static constexpr int CPS = PKSTEP / 8;                          // 16-byte chunks per row per step
-    // timing experiments only: 1 = no copies in the loop, 2 = copies from a fixed K offset,
-    // 4 = no operand reads in the loop.  (Per-workgroup timestamps are written whenever the
-    // launcher is given a trace buffer.)
+    // Timing experiments only (the library instantiates DBG = 0, which compiles none of it):
+    // 1 = no copies in the loop, 2 = copies from a fixed K offset, 4 = no operand reads in
+    // the loop; any non-zero value also records per-workgroup timestamps into `probe_out`.
     static constexpr int DBG = DBG_;
+    static constexpr int DBG_MODE = DBG_ & 7;
+    static constexpr bool TIMESTAMPS = DBG_ != 0;
     // Ring depths.  The B ring has STAGES buffers, the A ring STAGES + EXTRA_A: 256x256x64
     // tiles are 32 KB per operand and chunk, so the 160 KB of LDS hold two full stages plus
     // one more A buffer -- the A copies then run two chunks ahead and only the B copies
@@ -230,7 +232,7 @@ template <class Cfg, bool SPLIT = false, bool EDGE = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_pipelined_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
                            float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n,
-                           int first_block, int tail_tiles, int subdiv, long long *trace) {
+                           int first_block, int tail_tiles, int subdiv, long long *probe_out) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
     constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS, CPR = Cfg::CPR, CPS = Cfg::CPS;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES, SA = Cfg::SA, SB = Cfg::SB;
@@ -241,7 +243,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     static_assert(NFRAG <= NMMA, "at most one operand read is issued per MFMA slot");
     static_assert(!SPLIT || MI == 16, "fp32 partial stores are written for the 16x16x32 accumulator layout");
     long long t_begin = 0, t_loop = 0, t_epi = 0, c_loop = 0, c_epi = 0;
-    if (trace) t_begin = wall_clock64();
+    if constexpr (Cfg::TIMESTAMPS) t_begin = wall_clock64();
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
@@ -463,7 +465,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         const int nxt_b = (cur_b + 1 == SB) ? 0 : cur_b + 1;
         const int fill_a = (cur_a + FILL_OFF_A) % SA, fill_b = (cur_b + FILL_OFF_B) % SB;
         const unsigned char *a_src = a_next, *b_src = b_next;  // chunk kt + AHEAD
-        if constexpr (Cfg::DBG == 2) {
+        if constexpr (Cfg::DBG_MODE == 2) {
             a_src = a_base + (kt & 1) * BK * 2;
             b_src = b_base + (kt & 1) * BK * 2;
         }
@@ -492,13 +494,13 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             using SrcKK = std::integral_constant<int, (last ? 0 : kk + 1)>;
             static_for<NMMA>([&](auto idx_c) {
                 constexpr int idx = decltype(idx_c)::value;
-                constexpr int copy = (ISSUE && Cfg::DBG != 1 && Cfg::DBG != 4) ? copy_in_slot(kk * NMMA + idx) : -1;
+                constexpr int copy = (ISSUE && Cfg::DBG_MODE != 1 && Cfg::DBG_MODE != 4) ? copy_in_slot(kk * NMMA + idx) : -1;
                 if constexpr (copy >= 0)
                     mma_and_copy(idx_c, std::integral_constant<int, fb>{}, std::integral_constant<int, copy>{}, a_src,
                                  b_src, dst_a, dst_b);
                 else
                     mma_one(idx_c, std::integral_constant<int, fb>{});
-                if constexpr (prefetch && Cfg::DBG != 4) {
+                if constexpr (prefetch && Cfg::DBG_MODE != 4) {
                     // One operand read per slot at most, spread out (an LDS read in the slot
                     // right after another one stalls MFMA issue): A tile t for the next step
                     // at slot RS*t + 2, the double-buffered trailing B tiles at slots 0 and
@@ -518,10 +520,10 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             // Every operand read issued during this step has landed before control leaves
             // it.  The wait sits here, not at the top of the next step, so that no register
             // copy the compiler may place on a loop edge can see a fragment in flight.
-            if constexpr (prefetch && Cfg::DBG != 4) wait_operands(std::integral_constant<int, nb>{});
+            if constexpr (prefetch && Cfg::DBG_MODE != 4) wait_operands(std::integral_constant<int, nb>{});
         });
     };
-    if (trace) {
+    if constexpr (Cfg::TIMESTAMPS) {
         t_loop = wall_clock64();
         c_loop = clock64();
     }
@@ -561,7 +563,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         static_for<TN>([&](auto j_c) { pin_accumulator(acc[decltype(i_c)::value][decltype(j_c)::value]); });
     });
     // ---- epilogue: accumulators -> fp16 -> C (through LDS, whole lines per store)
-    if (trace) {
+    if constexpr (Cfg::TIMESTAMPS) {
         t_epi = wall_clock64();
         c_epi = clock64();
     }
@@ -593,9 +595,10 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         store_wave_tile<Cfg, Acc, EDGE>(acc, lds, C, M, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN,
                                         wave, lane);
     }
-    if (trace && tid == 0) {
+    if constexpr (Cfg::TIMESTAMPS) {
+      if (probe_out && tid == 0) {
         __builtin_amdgcn_s_waitcnt(0);
-        long long *t = trace + (size_t)blockIdx.x * 8;
+        long long *t = probe_out + (size_t)blockIdx.x * 8;
         t[0] = t_begin;
         t[1] = t_loop;
         t[2] = t_epi;
@@ -603,7 +606,9 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         t[4] = __builtin_amdgcn_s_getreg((31 << 11) | 4);   // HW_ID: wave / simd / cu / sh / se
         t[5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID
         t[6] = c_epi - c_loop;
+      }
     }
+    (void)t_begin, (void)t_loop, (void)t_epi, (void)c_loop, (void)c_epi, (void)probe_out;
 }
 
 // Shapes a pipelined kernel accepts with guarded edges: any M, N a multiple of 8 (rows of C
@@ -649,7 +654,7 @@ __global__ void __launch_bounds__(256)
 // as in the kernel.
 template <class Cfg, bool SPLIT, bool EDGE>
 void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial, size_t M, size_t N, size_t K,
-                           int splits, long long *trace, int first_block = 0, int blocks = -1, int tail_tiles = 0) {
+                           int splits, long long *probe_out, int first_block = 0, int blocks = -1, int tail_tiles = 0) {
     constexpr int subdiv = 0;
     static bool configured = [] {
         HGEMM_CHECK_HIP_ERROR(
@@ -663,7 +668,7 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
     HGEMM_CHECK(first_block >= 0 && blocks >= 1 && first_block + blocks <= tiles_m * tiles_n);
     hgemm_pipelined_kernel<Cfg, SPLIT, EDGE><<<dim3(blocks, splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), partial,
-        (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, first_block, tail_tiles, subdiv, trace);
+        (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, first_block, tail_tiles, subdiv, probe_out);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 
@@ -698,16 +703,16 @@ void launch_pipelined_with_tail(const void *A, const void *B, void *C, float *pa
 
 template <class Cfg>
 void launch_pipelined(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, const char *name,
-                      long long *trace = nullptr) {
+                      long long *probe_out = nullptr) {
     check_operands(A, B, C, M, N, K);
     if (Cfg::supports(M, N, K)) {
-        launch_pipelined_impl<Cfg, false, false>(A, B, C, nullptr, M, N, K, 1, trace);
+        launch_pipelined_impl<Cfg, false, false>(A, B, C, nullptr, M, N, K, 1, probe_out);
         return;
     }
     HGEMM_CHECK_MSG(pipelined_supports_edges<Cfg>(M, N, K),
                     "%s needs N %% 8 == 0, K %% %d == 0, K >= %d (got M=%zu N=%zu K=%zu)", name, Cfg::BK,
                     Cfg::BK * Cfg::STAGES, M, N, K);
-    launch_pipelined_impl<Cfg, false, true>(A, B, C, nullptr, M, N, K, 1, trace);
+    launch_pipelined_impl<Cfg, false, true>(A, B, C, nullptr, M, N, K, 1, probe_out);
 }
 
 // K split into `splits` slices: fp32 partial sums of slice s go to partial[s][M][N] (the

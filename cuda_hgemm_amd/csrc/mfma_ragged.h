@@ -33,7 +33,9 @@ __global__ void __launch_bounds__(RaggedConfig::THREADS)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * Cfg::BM, n0 = blockIdx.x * Cfg::BN;
+    // one-dimensional grid, row-major over the tiles of C: no 65535 limit on either dimension
+    const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
+    const int m0 = (int)(blockIdx.x / tiles_n) * Cfg::BM, n0 = (int)(blockIdx.x % tiles_n) * Cfg::BN;
     const int num_k = (K + BK - 1) / BK;
 
     // eight consecutive k of one row, zero where the row or k is outside the matrix
@@ -144,8 +146,7 @@ __global__ void __launch_bounds__(RaggedConfig::THREADS)
 
 inline void launch_ragged(const void *A, const void *B, void *C, size_t M, size_t N, size_t K) {
     check_operands(A, B, C, M, N, K);
-    const dim3 grid((unsigned)div_ceil(N, (size_t)RaggedConfig::BN), (unsigned)div_ceil(M, (size_t)RaggedConfig::BM));
-    HGEMM_CHECK_MSG(grid.y <= 65535u, "M=%zu needs more than 65535 row tiles", M);
+    const dim3 grid((unsigned)(div_ceil(N, (size_t)RaggedConfig::BN) * div_ceil(M, (size_t)RaggedConfig::BM)));
     const half_t *a = reinterpret_cast<const half_t *>(A), *b = reinterpret_cast<const half_t *>(B);
     half_t *c = reinterpret_cast<half_t *>(C);
     if (K % 8 == 0)

@@ -25,7 +25,7 @@ struct SkinnyConfig : TileConfig<BM_, BN_, 64, WAVES_M_, WAVES_N_, STAGES_, LOAD
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_skinny_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
-                        float *__restrict__ partial, int M, int N, int K, int k_per_split) {
+                        float *__restrict__ partial, int M, int N, int K, int k_per_split, int tiles_n) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, KSTEPS = Cfg::KSTEPS, CPR = Cfg::CPR;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES;
@@ -38,7 +38,8 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
 
-    const int tile_n = blockIdx.x, tile_m = blockIdx.y, split = blockIdx.z;
+    // grid: x = tiles of C, row-major (no 65535 limit on the number of row or column tiles), y = K slice
+    const int tile_n = (int)blockIdx.x % tiles_n, tile_m = (int)blockIdx.x / tiles_n, split = blockIdx.y;
     const int m0 = tile_m * BM;
     const int k_begin = split * k_per_split;
     const int num_k = k_per_split / BK;

@@ -92,6 +92,10 @@ __device__ __forceinline__ void wait_vmcnt() {
 // 1024 consecutive LDS bytes starting at the (wave-uniform) address in M0.  Written as
 // inline assembly so the compiler's wait-count insertion does not serialise LDS reads of
 // one stage behind copies into another; the kernel places its own s_waitcnt vmcnt(n).
+// M0 is written here without the compiler's knowledge (it is a reserved register: hipcc
+// warns that a clobber of it is not honoured).  gfx9 LDS instructions do not read M0 and
+// these kernels contain nothing else the compiler lowers through it (no indirect register
+// indexing, no compiler-generated LDS-DMA, no GWS), so nothing else depends on its value.
 __device__ __forceinline__ void dma_load16(const void *gptr, uint32_t lds_addr) {
     asm volatile(
         "s_mov_b32 m0, %0\n\t"

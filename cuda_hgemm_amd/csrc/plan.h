@@ -29,13 +29,30 @@ struct Plan {
     int kernel = KERNEL_NONE;
     int splits = 1;
     double est_us = 0.0;  // the cost model's estimate where it was used, else 0
+    // device memory the plan needs beyond A, B and C: fp32 partial sums of K slices, and
+    // zero-padded copies of unaligned operands (KERNEL_PADDED)
+    size_t partial_bytes = 0, operand_bytes = 0;
     // pipelined kernels only: the last tail_tiles workgroup ids of the grid run in tail_splits K slices, or
     // (tail_kernel != KERNEL_NONE, 256x256 tiles only) divided among workgroups of that smaller tile
     int tail_tiles = 0, tail_splits = 1, tail_kernel = KERNEL_NONE;
 };
 
+// Device memory handed to run_plan; a plan is only run with at least what it asks for.
+struct Workspace {
+    float *partial = nullptr;
+    size_t partial_bytes = 0;
+    unsigned char *operands = nullptr;
+    size_t operand_bytes = 0;
+};
+
+// Upper bounds on what a plan may ask for (0: plans that need no such memory only).
+struct PlanLimits {
+    size_t partial_bytes = 512ull << 20;
+    size_t operand_bytes = 1024ull << 20;
+};
+
 bool skinny_supports(size_t M, size_t N, size_t K);
-Plan plan_for(size_t M, size_t N, size_t K);
-void run_plan(const Plan &p, const void *A, const void *B, void *C, size_t M, size_t N, size_t K);
+Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits = PlanLimits());
+void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, void *C, size_t M, size_t N, size_t K);
 
 }  // namespace hgemm

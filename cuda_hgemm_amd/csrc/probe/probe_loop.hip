@@ -1,19 +1,25 @@
-// hgemm_probe_loop: where the time of the tuned 256x256x64 kernel goes, measured inside
-// the kernel.  The kernel is launched `launches` times back to back (the part settles on
+// hgemm_probe: where the time of the tuned 256x256x64 kernel goes, measured inside the
+// kernel.  A program of its own (bin/hgemm_probe), not part of libhgemm.so: the builds of
+// the kernel it runs carry timestamp code, and three of them compute nothing meaningful.  The kernel is launched `launches` times back to back (the part settles on
 // its power-limited clock only after some tens of launches); in the last launch one thread
-// per workgroup records wall-clock and shader-clock timestamps around its K loop.  Three
-// builds of the same kernel are available: the real one, one whose loop issues no
-// global -> LDS copies, and one that issues neither copies nor operand reads (their
-// results are meaningless; they exist to price the copies and the reads in issue slots and
-// in clock).
+// per workgroup records wall-clock and shader-clock timestamps around its K loop.  Four
+// builds of the same kernel are run: the real one, one whose copies always fetch the same
+// two K chunks (every copy hits L2: prices the traffic between L2 and the memory fabric),
+// one whose loop issues no global -> LDS copies, and one that issues neither copies nor
+// operand reads (the results of the last three are meaningless; they exist to price the
+// traffic, the copies and the reads in issue slots and in clock).
+//
+//     bin/hgemm_probe -M=8192 -N=8192 -K=8192 -launches=150
 #include <vector>
 
-#include "../../include/hgemm.h"
-#include "mfma_pipelined.h"
+#include "../driver/flags.h"
+#include "../driver/matrix.h"
+#include "../mfma_pipelined.h"
 
 namespace hgemm {
 namespace {
 
+// DBG 8: timestamps only; + 1: no copies; + 2: copies from a fixed K offset; + 4: no operand reads
 template <int DBG>
 using ProbeConfig = PipeConfig<256, 256, 64, 2, 2, 2, 16, 8, DBG, 1>;
 
@@ -32,7 +38,7 @@ void run_probe(const void *A, const void *B, void *C, size_t M, size_t N, size_t
     HGEMM_CHECK_HIP_ERROR(hipEventRecord(begin, nullptr));
     for (size_t i = 0; i < launches; ++i) {
         if (i + 1 == launches) HGEMM_CHECK_HIP_ERROR(hipEventRecord(last, nullptr));
-        launch_pipelined<Cfg>(A, B, C, M, N, K, "hgemm_probe_loop", i + 1 == launches ? trace : nullptr);
+        launch_pipelined<Cfg>(A, B, C, M, N, K, "hgemm_probe", i + 1 == launches ? trace : nullptr);
     }
     HGEMM_CHECK_HIP_ERROR(hipEventRecord(end, nullptr));
     HGEMM_CHECK_HIP_ERROR(hipEventSynchronize(end));
@@ -73,14 +79,33 @@ void run_probe(const void *A, const void *B, void *C, size_t M, size_t N, size_t
 }  // namespace
 }  // namespace hgemm
 
-extern "C" void hgemm_probe_loop(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K,
-                                 int mode, size_t launches, double *out8) {
+int main(int argc, char *argv[]) {
     using namespace hgemm;
-    HGEMM_CHECK(out8 != nullptr);
-    switch (mode) {
-        case 0: run_probe<0>(A, B, C, M, N, K, launches, out8); break;
-        case 1: run_probe<1>(A, B, C, M, N, K, launches, out8); break;
-        case 2: run_probe<4>(A, B, C, M, N, K, launches, out8); break;
-        default: HGEMM_CHECK_MSG(false, "probe mode %d (0: real kernel, 1: no copies, 2: no copies, no operand reads)", mode);
+    Flags flags;
+    flags.define("M", "8192", "M (a multiple of 256)");
+    flags.define("N", "8192", "N (a multiple of 256)");
+    flags.define("K", "8192", "K (a multiple of 64, at least 128)");
+    flags.define("launches", "150", "back-to-back launches per build; the last one is traced");
+    flags.define("seed", "20230212", "seed of the input matrices");
+    flags.parse(argc, argv);
+    const size_t M = flags.u64("M"), N = flags.u64("N"), K = flags.u64("K"), launches = flags.u64("launches");
+    const FillSpec uniform;
+    Matrix A(M, K, "Matrix A", flags.u64("seed"), 1, uniform), B(K, N, "Matrix B", flags.u64("seed"), 2, uniform);
+    Matrix C(M, N, "Matrix C", flags.u64("seed"), 3, FillSpec{Fill::Zero, 0.f, 0.f});
+    static const char *names[4] = {"tuned kernel", "copies always from the same two chunks (all L2 hits)",
+                                   "loop without copies", "loop without copies and operand reads"};
+    for (int mode = 0; mode < 4; ++mode) {
+        double r[8];
+        switch (mode) {
+            case 0: run_probe<8>(A.getDevPtr(), B.getDevPtr(), C.getDevPtr(), M, N, K, launches, r); break;
+            case 1: run_probe<8 + 2>(A.getDevPtr(), B.getDevPtr(), C.getDevPtr(), M, N, K, launches, r); break;
+            case 2: run_probe<8 + 1>(A.getDevPtr(), B.getDevPtr(), C.getDevPtr(), M, N, K, launches, r); break;
+            default: run_probe<8 + 4>(A.getDevPtr(), B.getDevPtr(), C.getDevPtr(), M, N, K, launches, r); break;
+        }
+        HLOG("Probe %s: %zu launches avg %.4f ms, traced launch %.4f ms (%.1f TFLOPS); per workgroup: prologue "
+             "%.2f us, loop %.2f us, epilogue %.2f us; loop %.0f shader cycles at %.3f GHz, MFMA issue %.1f%%",
+             names[mode], launches, r[0], r[1], 2.0 * M * N * K * 1e-12 / (r[1] * 1e-3), r[2], r[3], r[4], r[5], r[6],
+             100.0 * r[7]);
     }
+    return 0;
 }

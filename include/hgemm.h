@@ -16,8 +16,9 @@
  * fp16 once (the reference accumulates in fp16; this is the one deliberate difference).
  *
  * Calling convention, as in the reference (src/mma/mma_async_stage4.cu:637-644,
- * src/common/tester.h:59-62,91-94): launched asynchronously on the null stream, nothing is
- * allocated per call, the caller synchronises.  A contract violation (null pointer, zero
+ * src/common/tester.h:59-62,91-94): launched asynchronously on the null stream, the caller
+ * synchronises.  Nothing is allocated per call; hgemm_auto and hgemm_skinny allocate a
+ * process-lifetime workspace the first time a plan needs one (see "workspace" below).  A contract violation (null pointer, zero
  * dimension, a shape the variant cannot tile) is reported on stderr and ends the process
  * with EXIT_FAILURE, the convention of the reference's HGEMM_CHECK macros
  * (src/common/common.h:23-29); unlike the reference, unsupported shapes are diagnosed
@@ -80,6 +81,19 @@ HGEMM_FUNC(hgemm_mfma_async_stage2);
 HGEMM_FUNC(hgemm_mfma_async_stage3);
 HGEMM_FUNC(hgemm_mfma_async_stage4);
 
+/* The tuned CDNA4 kernel, one entry point per tile: K chunks of 64 in a ring of LDS buffers
+ * filled by direct-to-LDS copies, v_mfma_f32_16x16x32_f16 with a hand-laid issue order,
+ * XCD-aware tile order.  256x256 is the kernel hgemm_auto runs on large shapes and the top
+ * of the ladder, where the reference's run ends at mmaAsyncStage4 (reference
+ * src/main.cu:123, src/mma/mma_async_stage4.cu:637).  Need N % 8 == 0, K % 64 == 0 and
+ * K >= 64 * ring depth (128 / 192 / 192 / 320 / 192 in the order below); M and N may end
+ * inside a tile. */
+HGEMM_FUNC(hgemm_mfma_pipelined_256x256);
+HGEMM_FUNC(hgemm_mfma_pipelined_256x128);
+HGEMM_FUNC(hgemm_mfma_pipelined_192x192);
+HGEMM_FUNC(hgemm_mfma_pipelined_128x128);
+HGEMM_FUNC(hgemm_mfma_pipelined_64x64);
+
 /* Small-M (decode-shaped) product: streams B once, bound by HBM bandwidth, M <= 128.
  * No counterpart in the reference, whose tiled kernels cannot run M < 256
  * (reference src/mma/mma_async_stage4.cu:64-66,93-94). */
@@ -103,6 +117,27 @@ int hgemm_auto_plan_tail(size_t M, size_t N, size_t K, int *splits);
  * the plan does not do this; hgemm_auto_plan_tail still gives the number of tiles. */
 int hgemm_auto_plan_tail_kernel(size_t M, size_t N, size_t K);
 const char *hgemm_kernel_name(int kernel);
+
+/* ---- workspace of hgemm_auto / hgemm_skinny.  Plans that cut K into slices keep fp32
+ * partial sums in device memory, and large shapes with N % 8 != 0 or K % 64 != 0 run on
+ * zero-padded copies of A and B.  Both buffers belong to the library, one pair per device,
+ * and live until hgemm_release_workspace or the end of the process (the reference keeps its
+ * vendor handle the same way, src/cublas_tensor_op.cu:18).  Each is allocated ONCE, at its
+ * cap (512 MiB of partial sums, 1 GiB of operand copies), by the first call that needs it:
+ * that one call contains a hipMalloc; no later call allocates, frees or synchronises.
+ * Callers that cannot have even that (a timed loop, a stream being captured) reserve
+ * beforehand.  If the memory cannot be had, hgemm_auto runs the best plan that needs none.
+ * Entry points may be called from several host threads; the workspaces are shared, so
+ * calls that overlap on one device must be ordered on its null stream, as they are. */
+/* Allocates the current device's workspaces now: each at least as large as asked, and at
+ * least its cap, unless 0 is asked (that buffer is then left alone).  Returns 0, or 1 if
+ * device memory ran out. */
+int hgemm_reserve_workspace(size_t partial_bytes, size_t operand_bytes);
+/* Waits for the device and frees its workspaces. */
+void hgemm_release_workspace(void);
+/* Bytes of partial sums (return value) and of operand copies (*operand_bytes, if not NULL)
+ * that hgemm_auto's plan for the shape uses. */
+size_t hgemm_auto_workspace_bytes(size_t M, size_t N, size_t K, size_t *operand_bytes);
 
 /* ---- registry, so a driver can enumerate variants the way the reference's main lists
  * them (reference src/main.cu:100-123) without an edit per variant. ---- */
@@ -135,17 +170,6 @@ double hgemm_profile_rotating_ms(hgemm_fn fn, const hgemm_half *const *A, const 
 double hgemm_tflops(size_t M, size_t N, size_t K, double ms);
 /* Algorithmic bytes of one call: 2*(M*K + K*N + M*N). */
 double hgemm_bytes(size_t M, size_t N, size_t K);
-
-/* In-kernel timing of the tuned 256x256x64 kernel (M % 256 == N % 256 == 0, K % 64 == 0):
- * `launches` back-to-back launches, per-workgroup timestamps taken in the last one.
- * mode 0: the real kernel; 1: its loop without global->LDS copies; 2: without copies and
- * without operand reads (modes 1 and 2 leave garbage in C; they price the copies and the
- * reads).  out8 = { average ms per launch, ms of the traced launch, prologue us, loop us,
- * epilogue us (means per workgroup), shader cycles in the loop, shader clock in the loop
- * in GHz, fraction of the loop's cycles covered by the wave's MFMAs }.  No counterpart in
- * the reference (its profiling is done with ncu, run_sample.sh:23-27). */
-void hgemm_probe_loop(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K, int mode,
-                      size_t launches, double *out8);
 
 /* Library version string. */
 const char *hgemm_version(void);

@@ -47,6 +47,9 @@ def test_registry(hgemm_lib):
     variants = hgemm_lib.variants()
     names = [v["name"] for v in variants]
     assert names[0] == "Simt-Naive" and "Mfma-Async-Stage4" in names and names[-1] == "Auto"
+    # the tuned kernel is selectable by name and closes the ladder (reference src/main.cu:123)
+    assert names.index("Mfma-Pipelined-256x256") == names.index("Mfma-Async-Stage4") + 5
+    assert all(v["default_run"] for v in variants if v["name"].startswith("Mfma-Pipelined-"))
     assert len(set(names)) == len(names)
     for v in variants:
         assert hgemm_lib.find(v["name"]) == v["index"] == hgemm_lib.find(v["symbol"])
@@ -69,6 +72,13 @@ def test_shape_predicates(hgemm_lib):
         assert not s(name, 128, 128, 256) and not s(name, 256, 64, 256) and not s(name, 256, 128, 48)
     assert not s("hgemm_mfma_async_stage4", 256, 128, 64)      # K must cover the 3-chunk prologue
     assert s("hgemm_mfma_async_stage4", 256, 128, 96)
+    for name, ring in (("hgemm_mfma_pipelined_256x256", 2), ("hgemm_mfma_pipelined_256x128", 3),
+                       ("hgemm_mfma_pipelined_192x192", 3), ("hgemm_mfma_pipelined_128x128", 5),
+                       ("hgemm_mfma_pipelined_64x64", 3)):
+        assert s(name, 8192, 8192, 8192) and s(name, 1, 8, 64 * ring) and s(name, 1000, 4000, 1024)
+        assert not s(name, 256, 256, 64 * (ring - 1)) and not s(name, 256, 100, 1024) and not s(name, 256, 256, 1000)
+    # one-dimensional grids: no limit of 65535 row or column tiles
+    assert s("hgemm_auto", 4300000, 64, 64) and s("hgemm_simt_naive", 1100000, 16, 16)
     assert s("hgemm_skinny", 1, 4096, 4096) and s("hgemm_skinny", 128, 28672, 4096) and s("hgemm_skinny", 8, 192, 64)
     assert not s("hgemm_skinny", 129, 4096, 4096) and not s("hgemm_skinny", 8, 100, 4096)
     assert not s("hgemm_auto", 0, 8, 8) and not s("hgemm_auto", 1 << 20, 8, 1 << 20)
@@ -93,6 +103,24 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
     assert plan(100, 100, 100)["kernel"].startswith("guarded 128x128x32")      # no tile divides it
     assert plan(1000, 4000, 4096)["kernel"].startswith("pipelined")            # ragged M, N: guarded edges
     assert plan(4095, 4095, 4095)["kernel"].startswith("zero-padded")          # large and unaligned
+
+
+def test_workspace_needs_of_auto_plans(hgemm_lib):
+    """What hgemm_auto's plan keeps in device memory beyond A, B and C (no launch, no GPU)."""
+    need = hgemm_lib.auto_workspace_bytes
+    assert need(8192, 8192, 8192) == {"partial": 0, "operands": 0}
+    assert need(1, 4096, 4096) == {"partial": 0, "operands": 0}                 # one-launch decode kernel
+    p = hgemm_lib.auto_plan(256, 256, 16384)
+    assert p["splits"] > 1 and need(256, 256, 16384) == {"partial": p["splits"] * 256 * 256 * 4, "operands": 0}
+    p = hgemm_lib.auto_plan(64, 4096, 4096)
+    assert need(64, 4096, 4096)["partial"] == (p["splits"] * 64 * 4096 * 4 if p["splits"] > 1 else 0)
+    p = hgemm_lib.auto_plan(7168, 7168, 7168)                                    # last round in K slices
+    assert need(7168, 7168, 7168)["partial"] == p["tail_splits"] * p["tail_tiles"] * 256 * 256 * 4
+    padded = need(4095, 4095, 4095)                                             # A', B' and C' of 4095 x 4096 x 4096
+    assert padded["operands"] == 2 * (4095 * 4096 + 4096 * 4096 + 4095 * 4096)
+    for shape in ((16384, 16384, 16384), (100, 100, 100), (1 << 15, 1 << 15, 64)):
+        n = need(*shape)
+        assert n["partial"] <= 512 << 20 and n["operands"] <= 1024 << 20
 
 
 def test_metrics(hgemm_lib):

@@ -51,6 +51,8 @@ def _assert_close(oracle, got, ref_bits, K, ref_f32=None):
 
 TILED = ["hgemm_mfma_base", "hgemm_mfma_padding", "hgemm_mfma_swizzle", "hgemm_mfma_async", "hgemm_mfma_async_pg2s",
          "hgemm_mfma_async_pg2s_ps2r", "hgemm_mfma_async_stage2", "hgemm_mfma_async_stage3", "hgemm_mfma_async_stage4"]
+PIPELINED = ["hgemm_mfma_pipelined_64x64", "hgemm_mfma_pipelined_128x128", "hgemm_mfma_pipelined_192x192",
+             "hgemm_mfma_pipelined_256x128", "hgemm_mfma_pipelined_256x256"]
 ALL_AT_512 = ["hgemm_simt_naive", "hgemm_mfma_naive"] + TILED + ["hgemm_auto"]
 
 
@@ -115,6 +117,63 @@ def test_random_inputs_within_tolerance_and_deterministic(oracle, hgemm_lib, gpu
     assert np.array_equal(first, second), "results differ from run to run"
 
 
+# ------------------------------------------------------------------ the tuned kernel by tile, as named variants
+@pytest.mark.parametrize("variant", PIPELINED)
+@pytest.mark.parametrize("shape", [(256, 256, 320), (512, 2048, 1024), (300, 136, 384), (1000, 1000, 448)])
+def test_pipelined_variants(oracle, hgemm_lib, gpu, variant, shape):
+    """Every tile of the tuned kernel through its own entry point: the reference's checked
+    sample shape (run_sample.sh:60), the shortest K every ring accepts, and M, N ending inside a
+    tile.  Exact on ternary inputs, within tolerance and bit-identical run to run on random ones."""
+    M, N, K = shape
+    assert hgemm_lib.supports(variant, M, N, K)
+    At, Bt = oracle.fill((M, K), 51, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 51, 2, oracle.TERNARY, 0, 1)
+    assert np.array_equal(_run(hgemm_lib, variant, At, Bt, gpu), oracle.hgemm(At, Bt))
+    A, B = oracle.fill((M, K), 52, 1), oracle.fill((N, K), 52, 2)
+    first, second = _run(hgemm_lib, variant, A, B, gpu, repeat=2)
+    _assert_close(oracle, first, oracle.hgemm(A, B), K)
+    assert np.array_equal(first, second)
+
+
+@pytest.mark.parametrize("variant", PIPELINED)
+def test_pipelined_variants_identity_and_min_k(oracle, hgemm_lib, gpu, variant):
+    ring = {"64x64": 3, "128x128": 5, "192x192": 3, "256x128": 3, "256x256": 2}[variant.rsplit("_", 1)[1]]
+    K = 64 * ring
+    assert hgemm_lib.supports(variant, 256, 256, K) and not hgemm_lib.supports(variant, 256, 256, K - 64)
+    At, Bt = oracle.fill((256, K), 53, 1, oracle.TERNARY, 0, 1), oracle.fill((256, K), 53, 2, oracle.TERNARY, 0, 1)
+    assert np.array_equal(_run(hgemm_lib, variant, At, Bt, gpu), oracle.hgemm(At, Bt))
+    n = 384
+    eye = np.eye(n, dtype=np.float16).view(np.uint16)
+    B = oracle.fill((n, n), 7, 2)
+    assert np.array_equal(_run(hgemm_lib, variant, eye, B, gpu), B.T)
+
+
+def test_flagship_variant_is_the_kernel_auto_runs_at_8192(oracle, hgemm_lib, gpu):
+    n = 8192
+    assert hgemm_lib.auto_plan(n, n, n)["kernel"].startswith("pipelined 256x256x64")
+    A, B = oracle.fill((n, n), oracle.DEFAULT_SEED, 1), oracle.fill((n, n), oracle.DEFAULT_SEED, 2)
+    named = _run(hgemm_lib, "hgemm_mfma_pipelined_256x256", A, B, gpu)
+    assert np.array_equal(named, _run(hgemm_lib, "hgemm_auto", A, B, gpu))
+    _sampled_check(oracle, named, A, B, n, rows_per_slab=8, slabs=2)
+
+
+# ------------------------------------------------------------------ the ladder's rings at their shortest K
+@pytest.mark.parametrize("variant", TILED)
+def test_ladder_rings_at_minimum_k(oracle, hgemm_lib, gpu, variant):
+    """The shortest K each variant accepts (its prologue fills STAGES-1 buffers, so the loop
+    starts draining at once: the branch that waits for every copy from the first iteration
+    on), and one K chunk more."""
+    M, N = 512, 256
+    kmin = min(k for k in (32, 64, 96, 128, 160) if hgemm_lib.supports(variant, M, N, k))
+    expected = {"hgemm_mfma_async_stage2": 64, "hgemm_mfma_async_stage3": 64, "hgemm_mfma_async_stage4": 96}.get(variant, 32)
+    assert kmin == expected, (variant, kmin)
+    step = 64 if variant == "hgemm_mfma_async_stage2" else 32      # its K chunk is 64 wide
+    for K in (kmin, kmin + step):
+        At, Bt = oracle.fill((M, K), 61, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 61, 2, oracle.TERNARY, 0, 1)
+        assert np.array_equal(_run(hgemm_lib, variant, At, Bt, gpu), oracle.hgemm(At, Bt)), K
+        A, B = oracle.fill((M, K), 62, 1), oracle.fill((N, K), 62, 2)
+        _assert_close(oracle, _run(hgemm_lib, variant, A, B, gpu), oracle.hgemm(A, B), K)
+
+
 def test_vendor_comparator_matches_the_checker(oracle, vendor_lib, gpu):
     """Pins the transposes and leading dimensions of the hipBLASLt call."""
     import torch
@@ -154,6 +213,19 @@ def test_auto_large_shapes_sampled_rows(oracle, hgemm_lib, gpu, shape, dist_b):
         oracle.fill((N, K), oracle.DEFAULT_SEED, 2, oracle.NORMAL, 0.0, 0.02)
     first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
     _sampled_check(oracle, first, A, B, K)
+    assert np.array_equal(first, second)
+
+
+@pytest.mark.parametrize("n", [768, 1536, 3072, 5120, 7168, 15360])
+def test_auto_reference_sweep_dimensions(oracle, hgemm_lib, gpu, n):
+    """The squares of the reference's sweep (run_sample.sh:30) that are not benchmark
+    configurations, against the checker: whole matrix up to 1536, complete rows beyond."""
+    A, B = oracle.fill((n, n), oracle.DEFAULT_SEED, 1), oracle.fill((n, n), oracle.DEFAULT_SEED, 2)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    if n <= 1536:
+        _assert_close(oracle, first, oracle.hgemm(A, B), n)
+    else:
+        _sampled_check(oracle, first, A, B, n, rows_per_slab=8, slabs=4, seed=n)
     assert np.array_equal(first, second)
 
 
@@ -273,6 +345,38 @@ def test_auto_handles_shapes_no_tile_divides(oracle, hgemm_lib, gpu, shape):
     assert np.array_equal(first, second)
     At, Bt = oracle.fill((M, K), 14, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 14, 2, oracle.TERNARY, 0, 1)
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
+
+
+@pytest.mark.parametrize("variant,shape", [("hgemm_auto", (4300000, 64, 64)), ("hgemm_auto", (70000, 64, 128)),
+                                           ("hgemm_auto", (66000 * 128 + 5, 3, 5)), ("hgemm_simt_naive", (1100000, 16, 16)),
+                                           ("hgemm_simt_naive", (16, 1100000, 16)), ("hgemm_mfma_naive", (32, 2200000, 16)),
+                                           ("hgemm_mfma_naive", (2200000, 32, 16)), ("hgemm_auto", (8, 4300032, 64))])
+def test_more_row_or_column_tiles_than_a_grid_dimension_holds(oracle, hgemm_lib, gpu, variant, shape):
+    """Very tall or very wide outputs: more than 65535 tiles along M or N.  Every kernel
+    indexes its tiles through a one-dimensional grid, so these launch like any other shape."""
+    M, N, K = shape
+    assert hgemm_lib.supports(variant, M, N, K)
+    At, Bt = oracle.fill((M, K), 71, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 71, 2, oracle.TERNARY, 0, 1)
+    got = _run(hgemm_lib, variant, At, Bt, gpu)
+    ref = At.view(np.float16).astype(np.float32) @ Bt.view(np.float16).astype(np.float32).T   # exact: small integers
+    assert np.array_equal(got.view(np.float16).astype(np.float32), ref)
+
+
+def test_workspace_reserve_release_and_shape_changes(oracle, hgemm_lib, gpu):
+    """Shapes whose plans need growing amounts of partial sums and padded operand copies, in
+    turn, around an explicit reserve and release; results exact on ternary inputs."""
+    shapes = [(256, 256, 8192), (2048, 2048, 16384), (512, 512, 8192), (1111, 1111, 1111), (64, 4096, 4096),
+              (2047, 2049, 2051), (256, 256, 8192)]
+    need = [hgemm_lib.auto_workspace_bytes(*s) for s in shapes]
+    assert need[0]["partial"] > 0 and need[1]["partial"] > need[0]["partial"] and need[5]["operands"] > 0
+    hgemm_lib.release_workspace()
+    for round_ in range(2):
+        for (M, N, K) in shapes:
+            At, Bt = oracle.fill((M, K), 81, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 81, 2, oracle.TERNARY, 0, 1)
+            assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt)), (M, N, K)
+        if round_ == 0:
+            hgemm_lib.release_workspace()
+            hgemm_lib.reserve_workspace(1 << 20, 1 << 20)
 
 
 def test_guarded_edges_do_not_write_outside_c(oracle, hgemm_lib, gpu):

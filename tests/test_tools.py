@@ -36,6 +36,28 @@ def test_driver_command_uses_reference_flags():
     prof = benchmark.profiler_command(512, 2048, 1024, A)
     assert prof[0] == "rocprofv3" and prof[prof.index("--") + 1].endswith("bin/hgemm")
     assert "-profiling_iterations=1" in prof and A.iterations == 100
+    assert "--kernel-trace" in prof and "--pmc" not in prof
+
+
+def test_counter_sets_fit_one_pass_and_never_share_a_run_with_a_trace():
+    class A:
+        warmup, iterations, sleep_ms, check, naive, variant, json, out = 10, 100, 100, False, False, "Auto", False, "log"
+    assert set(benchmark.PMC_SETS) >= {"mfma", "lds", "fetch", "write"}
+    cost = {"FETCH_SIZE": ("TCC", 3), "WRITE_SIZE": ("TCC", 2)}
+    limit = {"SQ": 8, "TCC": 4, "TCP": 4, "TA": 2, "TD": 2, "GRBM": 2}
+    for name, counters in benchmark.PMC_SETS.items():
+        used = {}
+        for c in counters:
+            block, n = cost.get(c, (c.split("_")[0], 1))
+            used[block] = used.get(block, 0) + n
+        assert all(used[b] <= limit[b] for b in used), (name, used)
+        cmd = benchmark.profiler_command(8192, 8192, 8192, A, pmc=name)
+        body = cmd[:cmd.index("--")]
+        assert body[:2] == ["rocprofv3", "--pmc"] and body[2:2 + len(counters)] == counters
+        assert not any(flag in body for flag in ("--kernel-trace", "--stats", "--sys-trace", "-s", "--hip-trace",
+                                                 "--hsa-trace", "--memory-copy-trace", "--marker-trace", "-r"))
+        assert cmd[cmd.index("--") + 1].endswith("bin/hgemm") and f"rocprof_{name}" in " ".join(cmd)
+    assert benchmark.main(["--pmc", "nonsense", "--dims", "256"]) == 2
 
 
 def test_parse_and_tables(tmp_path):
