@@ -44,6 +44,7 @@ HELPER_SYMBOLS = [
     "hgemm_variant_fn", "hgemm_variant_find", "hgemm_variant_supports", "hgemm_variant_in_default_run",
     "hgemm_profile_ms", "hgemm_profile_rotating_ms", "hgemm_tflops", "hgemm_bytes", "hgemm_version",
     "hgemm_reserve_workspace", "hgemm_release_workspace", "hgemm_auto_workspace_bytes",
+    "hgemm_auto_static_workspace", "hgemm_static_workspace_bytes",
 ]
 
 
@@ -113,6 +114,8 @@ class HgemmLibrary:
         d.hgemm_release_workspace.argtypes, d.hgemm_release_workspace.restype = [], None
         d.hgemm_auto_workspace_bytes.argtypes = [_SZ, _SZ, _SZ, C.POINTER(_SZ)]
         d.hgemm_auto_workspace_bytes.restype = _SZ
+        d.hgemm_auto_static_workspace.argtypes, d.hgemm_auto_static_workspace.restype = _HGEMM_ARGS, C.c_int
+        d.hgemm_static_workspace_bytes.argtypes, d.hgemm_static_workspace_bytes.restype = [], _SZ
 
     # ---- registry -------------------------------------------------------------------
     def variants(self) -> List[dict]:
@@ -152,6 +155,9 @@ class HgemmLibrary:
 
     def release_workspace(self) -> None:
         self.dll.hgemm_release_workspace()
+
+    def static_workspace_bytes(self) -> int:
+        return self.dll.hgemm_static_workspace_bytes()
 
     def version(self) -> str:
         return self.dll.hgemm_version().decode()

@@ -66,6 +66,26 @@ bool heap_workspace(size_t partial_bytes, size_t operand_bytes, Workspace *out) 
     return ok;
 }
 
+// Scratch of the entry point that allocates nothing: a fixed array in the code object, one
+// copy per device, partial sums first and padded operands behind them.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; kernels get the device address.
+constexpr size_t STATIC_WORKSPACE_BYTES = HGEMM_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_WORKSPACE_BYTES];
+std::mutex g_scratch_mutex;
+unsigned char *g_scratch_ptr[MAX_DEVICES];
+
+unsigned char *static_scratch() {
+    const int dev = current_device();
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        HGEMM_CHECK_HIP_ERROR(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        HGEMM_CHECK(ptr != nullptr);
+        g_scratch_ptr[dev] = reinterpret_cast<unsigned char *>(ptr);
+    }
+    return g_scratch_ptr[dev];
+}
+
 int compute_units() {
     static int cus = [] {
         // A planning query must also work where no GPU is visible: assume one MI355X.
@@ -537,6 +557,33 @@ extern "C" void hgemm_release_workspace(void) {
     if (w.operands) HGEMM_CHECK_HIP_ERROR(hipFree(w.operands));
     w = Workspace();
 }
+
+extern "C" int hgemm_auto_static_workspace(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N,
+                                           size_t K) {
+    check_operands(A, B, C, M, N, K);
+    const Plan &p = cached_plan(M, N, K);  // the plan hgemm_auto runs: same kernels, same order of additions
+    const size_t partial_bytes = (p.partial_bytes + 255) / 256 * 256;
+    if (partial_bytes + p.operand_bytes > STATIC_WORKSPACE_BYTES) {
+        HLOG("hgemm_auto_static_workspace: the plan for M=%zu N=%zu K=%zu keeps %zu bytes of partial sums and %zu bytes "
+             "of padded operands, the static workspace holds %zu; nothing was launched (hgemm_auto has no such limit)",
+             M, N, K, p.partial_bytes, p.operand_bytes, STATIC_WORKSPACE_BYTES);
+        return 1;
+    }
+    Workspace ws;
+    if (partial_bytes + p.operand_bytes > 0) {
+        unsigned char *base = static_scratch();
+        ws.partial = reinterpret_cast<float *>(base);
+        ws.partial_bytes = partial_bytes;
+        ws.operands = base + partial_bytes;
+        ws.operand_bytes = STATIC_WORKSPACE_BYTES - partial_bytes;
+    }
+    // Nothing in the array has to start at zero: every kernel that reads partial sums or padded
+    // operands reads only what a kernel launched before it in this call has written in full.
+    run_plan(p, ws, A, B, C, M, N, K);
+    return 0;
+}
+
+extern "C" size_t hgemm_static_workspace_bytes(void) { return STATIC_WORKSPACE_BYTES; }
 
 extern "C" size_t hgemm_auto_workspace_bytes(size_t M, size_t N, size_t K, size_t *operand_bytes) {
     const Plan p = plan_for(M, N, K);

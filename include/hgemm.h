@@ -139,6 +139,21 @@ void hgemm_release_workspace(void);
  * that hgemm_auto's plan for the shape uses. */
 size_t hgemm_auto_workspace_bytes(size_t M, size_t N, size_t K, size_t *operand_bytes);
 
+/* hgemm_auto for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Runs
+ * the same plan as hgemm_auto, hence the same result bit for bit, but keeps partial sums and
+ * padded operand copies in a fixed array of HGEMM_STATIC_WORKSPACE_BYTES inside the library's
+ * code object (every GPU the library runs on holds one copy until the process ends) and
+ * calls no hipMalloc, hipFree or other allocating routine.  Returns 0, or 1 -- with a
+ * message on stderr and nothing launched -- when the plan needs more than the array holds
+ * (hgemm_auto_workspace_bytes tells beforehand).  Other contract violations end the process
+ * as everywhere.  All calls on one GPU share that GPU's array: calls that overlap on a GPU
+ * (different streams or host threads) race; calls on the null stream are ordered. */
+#define HGEMM_STATIC_WORKSPACE_BYTES ((size_t)64 << 20)
+int hgemm_auto_static_workspace(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N,
+                                size_t K);
+size_t hgemm_static_workspace_bytes(void);
+
 /* ---- registry, so a driver can enumerate variants the way the reference's main lists
  * them (reference src/main.cu:100-123) without an edit per variant. ---- */
 int hgemm_variant_count(void);
