@@ -37,7 +37,8 @@ KERNEL_SYMBOLS = [
     "hgemm_mfma_async", "hgemm_mfma_async_pg2s", "hgemm_mfma_async_pg2s_ps2r", "hgemm_mfma_async_stage2",
     "hgemm_mfma_async_stage3", "hgemm_mfma_async_stage4", "hgemm_mfma_pipelined_64x64",
     "hgemm_mfma_pipelined_128x128", "hgemm_mfma_pipelined_192x192", "hgemm_mfma_pipelined_256x128",
-    "hgemm_mfma_pipelined_256x256", "hgemm_skinny", "hgemm_auto",
+    "hgemm_mfma_pipelined_256x256", "hgemm_mfma_chained_192x192", "hgemm_mfma_chained_256x128",
+    "hgemm_mfma_chained_256x256", "hgemm_skinny", "hgemm_auto",
 ]
 HELPER_SYMBOLS = [
     "hgemm_auto_plan", "hgemm_auto_plan_tail", "hgemm_auto_plan_tail_kernel", "hgemm_kernel_name", "hgemm_variant_count", "hgemm_variant_name", "hgemm_variant_symbol",

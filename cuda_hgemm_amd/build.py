@@ -61,8 +61,9 @@ def _run(cmd):
 
 # Kernels whose operands and accumulators are handled from inline assembly in an order the
 # compiler does not know: a register spill between an LDS read and its wait, or of an
-# accumulator, would corrupt results silently, so the build fails if one appears.
-NO_SPILL_KERNELS = ("hgemm_pipelined_kernel",)
+# accumulator, would corrupt results silently, and the chained kernel keeps its accumulators
+# in AGPRs the compiler must never look for, so the build fails if a spill appears.
+NO_SPILL_KERNELS = ("hgemm_pipelined_kernel", "hgemm_chained_kernel")
 
 
 def _check_no_spills(src, remarks):

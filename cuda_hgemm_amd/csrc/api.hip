@@ -17,6 +17,9 @@ HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_128x128);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_192x192);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_256x128);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_256x256);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_chained_192x192);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_chained_256x128);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_chained_256x256);
 HGEMM_DECLARE_SUPPORTS(hgemm_skinny);
 HGEMM_DECLARE_SUPPORTS(hgemm_auto);
 
@@ -60,6 +63,13 @@ const Variant kVariants[] = {
      hgemm_mfma_pipelined_256x128_supports, 1},
     {"Mfma-Pipelined-256x256", "hgemm_mfma_pipelined_256x256", hgemm_mfma_pipelined_256x256,
      hgemm_mfma_pipelined_256x256_supports, 1},
+    // the last rung: each accumulator's MFMAs back to back
+    {"Mfma-Chained-192x192", "hgemm_mfma_chained_192x192", hgemm_mfma_chained_192x192,
+     hgemm_mfma_chained_192x192_supports, 1},
+    {"Mfma-Chained-256x128", "hgemm_mfma_chained_256x128", hgemm_mfma_chained_256x128,
+     hgemm_mfma_chained_256x128_supports, 1},
+    {"Mfma-Chained-256x256", "hgemm_mfma_chained_256x256", hgemm_mfma_chained_256x256,
+     hgemm_mfma_chained_256x256_supports, 1},
     {"Skinny", "hgemm_skinny", hgemm_skinny, hgemm_skinny_supports, 1},
     {"Auto", "hgemm_auto", hgemm_auto, hgemm_auto_supports, 1},
 };

@@ -529,19 +529,23 @@ extern "C" void hgemm_auto(const hgemm_half *A, const hgemm_half *B, hgemm_half 
 }
 
 // The tuned kernel by tile, as entry points of their own.  M and N may end inside a tile.
-#define HGEMM_DEFINE_PIPELINED_VARIANT(symbol, Cfg)                                                          \
+#define HGEMM_DEFINE_PIPELINED_VARIANT(symbol, Cfg, which)                                                   \
     extern "C" void symbol(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N,      \
                            size_t K) {                                                                       \
-        launch_pipelined<Cfg>(A, B, C, M, N, K, #symbol);                                                    \
+        launch_pipelined<Cfg>(A, B, C, M, N, K, #symbol, nullptr, which);                                    \
     }                                                                                                        \
     extern "C" int symbol##_supports(size_t M, size_t N, size_t K) {                                         \
         return pipelined_supports_edges<Cfg>(M, N, K) ? 1 : 0;                                               \
     }
-HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_64x64, Small64)
-HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_128x128, Mid128)
-HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_192x192, Tile192)
-HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_256x128, Rect256x128)
-HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_256x256, Big256)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_64x64, Small64, PipeKernel::Interleaved)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_128x128, Mid128, PipeKernel::Interleaved)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_192x192, Tile192, PipeKernel::Interleaved)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_256x128, Rect256x128, PipeKernel::Interleaved)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_pipelined_256x256, Big256, PipeKernel::Interleaved)
+// ... and with each accumulator's MFMAs chained (the tiles that have that kernel)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_chained_192x192, Tile192, PipeKernel::Chained)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_chained_256x128, Rect256x128, PipeKernel::Chained)
+HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_chained_256x256, Big256, PipeKernel::Chained)
 
 extern "C" int hgemm_reserve_workspace(size_t partial_bytes, size_t operand_bytes) {
     Workspace ws;

@@ -1,5 +1,5 @@
-// hgemm_probe: where the time of the tuned 256x256x64 kernel goes, measured inside the
-// kernel.  A program of its own (bin/hgemm_probe), not part of libhgemm.so: the builds of
+// hgemm_probe: where the time of the tuned 256x256x64 kernels (interleaved and chained) goes,
+// measured inside the kernel.  A program of its own (bin/hgemm_probe), not part of libhgemm.so: the builds of
 // the kernel it runs carry timestamp code, and three of them compute nothing meaningful.  The kernel is launched `launches` times back to back (the part settles on
 // its power-limited clock only after some tens of launches); in the last launch one thread
 // per workgroup records wall-clock and shader-clock timestamps around its K loop.  Four
@@ -23,7 +23,7 @@ namespace {
 template <int DBG>
 using ProbeConfig = PipeConfig<256, 256, 64, 2, 2, 2, 16, 8, DBG, 1>;
 
-template <int DBG>
+template <int DBG, PipeKernel WHICH = PipeKernel::Interleaved>
 void run_probe(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, size_t launches, double *out) {
     using Cfg = ProbeConfig<DBG>;
     HGEMM_CHECK_MSG(Cfg::supports(M, N, K), "the probe needs M %% 256 == 0, N %% 256 == 0, K %% 64 == 0, K >= 128");
@@ -38,7 +38,7 @@ void run_probe(const void *A, const void *B, void *C, size_t M, size_t N, size_t
     HGEMM_CHECK_HIP_ERROR(hipEventRecord(begin, nullptr));
     for (size_t i = 0; i < launches; ++i) {
         if (i + 1 == launches) HGEMM_CHECK_HIP_ERROR(hipEventRecord(last, nullptr));
-        launch_pipelined<Cfg>(A, B, C, M, N, K, "hgemm_probe", i + 1 == launches ? trace : nullptr);
+        launch_pipelined<Cfg>(A, B, C, M, N, K, "hgemm_probe", i + 1 == launches ? trace : nullptr, WHICH);
     }
     HGEMM_CHECK_HIP_ERROR(hipEventRecord(end, nullptr));
     HGEMM_CHECK_HIP_ERROR(hipEventSynchronize(end));
@@ -92,15 +92,24 @@ int main(int argc, char *argv[]) {
     const FillSpec uniform;
     Matrix A(M, K, "Matrix A", flags.u64("seed"), 1, uniform), B(K, N, "Matrix B", flags.u64("seed"), 2, uniform);
     Matrix C(M, N, "Matrix C", flags.u64("seed"), 3, FillSpec{Fill::Zero, 0.f, 0.f});
-    static const char *names[4] = {"tuned kernel", "copies always from the same two chunks (all L2 hits)",
-                                   "loop without copies", "loop without copies and operand reads"};
-    for (int mode = 0; mode < 4; ++mode) {
+    static const char *names[8] = {"interleaved kernel", "interleaved, copies always from the same two chunks (all L2 hits)",
+                                   "interleaved, loop without copies", "interleaved, loop without copies and operand reads",
+                                   "chained kernel", "chained, copies always from the same two chunks (all L2 hits)",
+                                   "chained, loop without copies", "chained, loop without copies and operand reads"};
+    constexpr PipeKernel CH = PipeKernel::Chained;
+    for (int mode = 0; mode < 8; ++mode) {
         double r[8];
+        const uint16_t *a = A.getDevPtr(), *b = B.getDevPtr();
+        uint16_t *c = C.getDevPtr();
         switch (mode) {
-            case 0: run_probe<8>(A.getDevPtr(), B.getDevPtr(), C.getDevPtr(), M, N, K, launches, r); break;
-            case 1: run_probe<8 + 2>(A.getDevPtr(), B.getDevPtr(), C.getDevPtr(), M, N, K, launches, r); break;
-            case 2: run_probe<8 + 1>(A.getDevPtr(), B.getDevPtr(), C.getDevPtr(), M, N, K, launches, r); break;
-            default: run_probe<8 + 4>(A.getDevPtr(), B.getDevPtr(), C.getDevPtr(), M, N, K, launches, r); break;
+            case 0: run_probe<8>(a, b, c, M, N, K, launches, r); break;
+            case 1: run_probe<8 + 2>(a, b, c, M, N, K, launches, r); break;
+            case 2: run_probe<8 + 1>(a, b, c, M, N, K, launches, r); break;
+            case 3: run_probe<8 + 4>(a, b, c, M, N, K, launches, r); break;
+            case 4: run_probe<8, CH>(a, b, c, M, N, K, launches, r); break;
+            case 5: run_probe<8 + 2, CH>(a, b, c, M, N, K, launches, r); break;
+            case 6: run_probe<8 + 1, CH>(a, b, c, M, N, K, launches, r); break;
+            default: run_probe<8 + 4, CH>(a, b, c, M, N, K, launches, r); break;
         }
         HLOG("Probe %s: %zu launches avg %.4f ms, traced launch %.4f ms (%.1f TFLOPS); per workgroup: prologue "
              "%.2f us, loop %.2f us, epilogue %.2f us; loop %.0f shader cycles at %.3f GHz, MFMA issue %.1f%%",

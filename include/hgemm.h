@@ -93,6 +93,14 @@ HGEMM_FUNC(hgemm_mfma_pipelined_256x128);
 HGEMM_FUNC(hgemm_mfma_pipelined_192x192);
 HGEMM_FUNC(hgemm_mfma_pipelined_128x128);
 HGEMM_FUNC(hgemm_mfma_pipelined_64x64);
+/* The same tiles with the work inside a K chunk reordered so that every accumulator receives
+ * its two MFMAs back to back (the matrix pipe forwards the running sum instead of going
+ * through the register file: less power, hence more clock) and with the accumulators in
+ * registers the compiler never sees.  The top of the ladder; hgemm_auto runs these on large
+ * shapes with K >= 3072.  Same shape needs as the pipelined entry points above. */
+HGEMM_FUNC(hgemm_mfma_chained_256x256);
+HGEMM_FUNC(hgemm_mfma_chained_256x128);
+HGEMM_FUNC(hgemm_mfma_chained_192x192);
 
 /* Small-M (decode-shaped) product: streams B once, bound by HBM bandwidth, M <= 128.
  * No counterpart in the reference, whose tiled kernels cannot run M < 256

@@ -49,7 +49,8 @@ def test_registry(hgemm_lib):
     assert names[0] == "Simt-Naive" and "Mfma-Async-Stage4" in names and names[-1] == "Auto"
     # the tuned kernel is selectable by name and closes the ladder (reference src/main.cu:123)
     assert names.index("Mfma-Pipelined-256x256") == names.index("Mfma-Async-Stage4") + 5
-    assert all(v["default_run"] for v in variants if v["name"].startswith("Mfma-Pipelined-"))
+    assert names.index("Mfma-Chained-256x256") == names.index("Mfma-Pipelined-256x256") + 3 == len(names) - 3
+    assert all(v["default_run"] for v in variants if v["name"].startswith(("Mfma-Pipelined-", "Mfma-Chained-")))
     assert len(set(names)) == len(names)
     for v in variants:
         assert hgemm_lib.find(v["name"]) == v["index"] == hgemm_lib.find(v["symbol"])
@@ -74,7 +75,8 @@ def test_shape_predicates(hgemm_lib):
     assert s("hgemm_mfma_async_stage4", 256, 128, 96)
     for name, ring in (("hgemm_mfma_pipelined_256x256", 2), ("hgemm_mfma_pipelined_256x128", 3),
                        ("hgemm_mfma_pipelined_192x192", 3), ("hgemm_mfma_pipelined_128x128", 5),
-                       ("hgemm_mfma_pipelined_64x64", 3)):
+                       ("hgemm_mfma_pipelined_64x64", 3), ("hgemm_mfma_chained_256x256", 2),
+                       ("hgemm_mfma_chained_256x128", 3), ("hgemm_mfma_chained_192x192", 3)):
         assert s(name, 8192, 8192, 8192) and s(name, 1, 8, 64 * ring) and s(name, 1000, 4000, 1024)
         assert not s(name, 256, 256, 64 * (ring - 1)) and not s(name, 256, 100, 1024) and not s(name, 256, 256, 1000)
     # one-dimensional grids: no limit of 65535 row or column tiles

@@ -52,7 +52,8 @@ def _assert_close(oracle, got, ref_bits, K, ref_f32=None):
 TILED = ["hgemm_mfma_base", "hgemm_mfma_padding", "hgemm_mfma_swizzle", "hgemm_mfma_async", "hgemm_mfma_async_pg2s",
          "hgemm_mfma_async_pg2s_ps2r", "hgemm_mfma_async_stage2", "hgemm_mfma_async_stage3", "hgemm_mfma_async_stage4"]
 PIPELINED = ["hgemm_mfma_pipelined_64x64", "hgemm_mfma_pipelined_128x128", "hgemm_mfma_pipelined_192x192",
-             "hgemm_mfma_pipelined_256x128", "hgemm_mfma_pipelined_256x256"]
+             "hgemm_mfma_pipelined_256x128", "hgemm_mfma_pipelined_256x256", "hgemm_mfma_chained_192x192",
+             "hgemm_mfma_chained_256x128", "hgemm_mfma_chained_256x256"]
 ALL_AT_512 = ["hgemm_simt_naive", "hgemm_mfma_naive"] + TILED + ["hgemm_auto"]
 
 
@@ -119,11 +120,14 @@ def test_random_inputs_within_tolerance_and_deterministic(oracle, hgemm_lib, gpu
 
 # ------------------------------------------------------------------ the tuned kernel by tile, as named variants
 @pytest.mark.parametrize("variant", PIPELINED)
-@pytest.mark.parametrize("shape", [(256, 256, 320), (512, 2048, 1024), (300, 136, 384), (1000, 1000, 448)])
+@pytest.mark.parametrize("shape", [(256, 256, 320), (512, 2048, 1024), (300, 136, 384), (1000, 1000, 448),
+                                   (768, 512, 3072), (520, 776, 3136)])
 def test_pipelined_variants(oracle, hgemm_lib, gpu, variant, shape):
-    """Every tile of the tuned kernel through its own entry point: the reference's checked
-    sample shape (run_sample.sh:60), the shortest K every ring accepts, and M, N ending inside a
-    tile.  Exact on ternary inputs, within tolerance and bit-identical run to run on random ones."""
+    """Every tile of the tuned kernel through its own entry point, interleaved and chained: the
+    reference's checked sample shape (run_sample.sh:60), the shortest K every ring accepts, M and
+    N ending inside a tile, K of 5, 6, 7, 16, 48 and 49 chunks (the chained kernel's unrolled loop
+    covers six chunks per trip, the rest go through its loop with run-time ring indices).
+    Exact on ternary inputs, within tolerance and bit-identical run to run on random ones."""
     M, N, K = shape
     assert hgemm_lib.supports(variant, M, N, K)
     At, Bt = oracle.fill((M, K), 51, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 51, 2, oracle.TERNARY, 0, 1)
@@ -148,11 +152,14 @@ def test_pipelined_variants_identity_and_min_k(oracle, hgemm_lib, gpu, variant):
 
 
 def test_flagship_variant_is_the_kernel_auto_runs_at_8192(oracle, hgemm_lib, gpu):
+    """The top rung by name; the interleaved kernel on the same tile adds every output's products
+    in the same order, so all three agree bit for bit."""
     n = 8192
     assert hgemm_lib.auto_plan(n, n, n)["kernel"].startswith("pipelined 256x256x64")
     A, B = oracle.fill((n, n), oracle.DEFAULT_SEED, 1), oracle.fill((n, n), oracle.DEFAULT_SEED, 2)
-    named = _run(hgemm_lib, "hgemm_mfma_pipelined_256x256", A, B, gpu)
+    named = _run(hgemm_lib, "hgemm_mfma_chained_256x256", A, B, gpu)
     assert np.array_equal(named, _run(hgemm_lib, "hgemm_auto", A, B, gpu))
+    assert np.array_equal(named, _run(hgemm_lib, "hgemm_mfma_pipelined_256x256", A, B, gpu))
     _sampled_check(oracle, named, A, B, n, rows_per_slab=8, slabs=2)
 
 
