@@ -41,7 +41,7 @@ KERNEL_SYMBOLS = [
     "hgemm_mfma_chained_256x256", "hgemm_skinny", "hgemm_auto",
 ]
 HELPER_SYMBOLS = [
-    "hgemm_auto_plan", "hgemm_auto_plan_tail", "hgemm_auto_plan_tail_kernel", "hgemm_kernel_name", "hgemm_variant_count", "hgemm_variant_name", "hgemm_variant_symbol",
+    "hgemm_auto_plan", "hgemm_auto_plan_tail", "hgemm_auto_plan_tail_kernel", "hgemm_auto_plan_chained", "hgemm_kernel_name", "hgemm_variant_count", "hgemm_variant_name", "hgemm_variant_symbol",
     "hgemm_variant_fn", "hgemm_variant_find", "hgemm_variant_supports", "hgemm_variant_in_default_run",
     "hgemm_profile_ms", "hgemm_profile_rotating_ms", "hgemm_tflops", "hgemm_bytes", "hgemm_version",
     "hgemm_reserve_workspace", "hgemm_release_workspace", "hgemm_auto_workspace_bytes",
@@ -95,6 +95,7 @@ class HgemmLibrary:
         d.hgemm_auto_plan.argtypes, d.hgemm_auto_plan.restype = [_SZ, _SZ, _SZ, C.POINTER(C.c_int)], C.c_int
         d.hgemm_auto_plan_tail.argtypes, d.hgemm_auto_plan_tail.restype = [_SZ, _SZ, _SZ, C.POINTER(C.c_int)], C.c_int
         d.hgemm_auto_plan_tail_kernel.argtypes, d.hgemm_auto_plan_tail_kernel.restype = [_SZ, _SZ, _SZ], C.c_int
+        d.hgemm_auto_plan_chained.argtypes, d.hgemm_auto_plan_chained.restype = [_SZ, _SZ, _SZ], C.c_int
         d.hgemm_kernel_name.argtypes, d.hgemm_kernel_name.restype = [C.c_int], C.c_char_p
         d.hgemm_variant_count.argtypes, d.hgemm_variant_count.restype = [], C.c_int
         d.hgemm_variant_name.argtypes, d.hgemm_variant_name.restype = [C.c_int], C.c_char_p
@@ -142,6 +143,7 @@ class HgemmLibrary:
         tail_splits = C.c_int(1)
         tail_tiles = self.dll.hgemm_auto_plan_tail(M, N, K, C.byref(tail_splits))
         return {"kernel_id": kernel, "kernel": self.dll.hgemm_kernel_name(kernel).decode(), "splits": splits.value,
+                "chained": bool(self.dll.hgemm_auto_plan_chained(M, N, K)),
                 "tail_tiles": tail_tiles, "tail_splits": tail_splits.value,
                 "tail_kernel": self.dll.hgemm_kernel_name(self.dll.hgemm_auto_plan_tail_kernel(M, N, K)).decode()}
 

@@ -3,7 +3,8 @@
     cuda_hgemm_amd/lib/libhgemm.so            the kernels + C ABI (include/hgemm.h)
     cuda_hgemm_amd/lib/libhgemm_hipblaslt.so  vendor comparator (include/hgemm_hipblaslt.h)
     cuda_hgemm_amd/bin/hgemm                  C++ benchmark / check driver
-    cuda_hgemm_amd/bin/hgemm_probe            in-kernel timing of the tuned kernel (evidence tool)
+    cuda_hgemm_amd/bin/hgemm_probe            in-kernel timing of the tuned kernels (evidence tool)
+    cuda_hgemm_amd/bin/hgemm_mix_probe        cost of each piece of their loop under the power limit (evidence tool)
 
 Run as ``python -m cuda_hgemm_amd.build`` (add ``--force`` to rebuild everything).
 hipcc cross-compiles without a GPU, so this works on a CPU-only machine.
@@ -33,7 +34,9 @@ LIB_SOURCES = ["basic_kernels.hip", "ladder_sync.hip", "ladder_async.hip", "ladd
                "api.hip"]
 VENDOR_SOURCES = ["vendor_hipblaslt.cpp"]
 DRIVER_SOURCES = ["driver/main.cpp"]
-PROBE_SOURCES = ["probe/probe_loop.hip"]   # bin/hgemm_probe: in-kernel timing, not part of the library
+# evidence tools, not part of the library: bin/hgemm_probe (in-kernel timing of the tuned kernels)
+# and bin/hgemm_mix_probe (what each piece of their loop costs under the power limit)
+PROBE_SOURCES = ["probe/probe_loop.hip", "probe/issue_mix.hip"]
 
 
 def _headers():
@@ -123,13 +126,14 @@ def build(force: bool = False, verbose: bool = False) -> dict:
     if force or _stale(driver, drv_objs + [libhgemm, vendor]):
         _run([HIPCC, "-o", driver] + drv_objs + ["-L" + LIB, "-lhgemm", "-lhgemm_hipblaslt", "-fopenmp",
                                                   "-Wl,-rpath,$ORIGIN/../lib"])
-    probe = os.path.join(BIN, "hgemm_probe")
-    probe_objs = [objs[s] for s in PROBE_SOURCES]
-    if force or _stale(probe, probe_objs):
-        _run([HIPCC, "-o", probe] + probe_objs + ["-fopenmp"])
+    probes = {}
+    for src, name in zip(PROBE_SOURCES, ("hgemm_probe", "hgemm_mix_probe")):
+        probes[name] = os.path.join(BIN, name)
+        if force or _stale(probes[name], [objs[src]]):
+            _run([HIPCC, "-o", probes[name], objs[src], "-fopenmp"])
     if verbose:
-        print("built", libhgemm, vendor, driver, probe)
-    return {"libhgemm": libhgemm, "vendor": vendor, "driver": driver, "probe": probe}
+        print("built", libhgemm, vendor, driver, *probes.values())
+    return {"libhgemm": libhgemm, "vendor": vendor, "driver": driver, **probes}
 
 
 if __name__ == "__main__":

@@ -611,6 +611,18 @@ extern "C" int hgemm_auto_plan_tail(size_t M, size_t N, size_t K, int *splits) {
 }
 // Kernel id of the smaller tile that takes over the last round (0: none).
 extern "C" int hgemm_auto_plan_tail_kernel(size_t M, size_t N, size_t K) { return plan_for(M, N, K).tail_kernel; }
+// 1 if the plan's main launch runs the chained kernel of its tile, 0 for the interleaved one.
+extern "C" int hgemm_auto_plan_chained(size_t M, size_t N, size_t K) {
+    const Plan p = plan_for(M, N, K);
+    if (p.splits < 1) return 0;
+    const size_t k_len = K / (size_t)p.splits;
+    switch (p.kernel) {
+        case KERNEL_BIG256: return use_chained<Big256>(PipeKernel::Auto, k_len) ? 1 : 0;
+        case KERNEL_T192: return use_chained<Tile192>(PipeKernel::Auto, k_len) ? 1 : 0;
+        case KERNEL_R256x128: return use_chained<Rect256x128>(PipeKernel::Auto, k_len) ? 1 : 0;
+        default: return 0;
+    }
+}
 extern "C" const char *hgemm_kernel_name(int kernel) {
     switch (kernel) {
         case KERNEL_BIG256: return "pipelined 256x256x64, 4 waves, LDS ring 3 (A) + 2 (B)";

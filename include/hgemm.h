@@ -124,6 +124,9 @@ int hgemm_auto_plan_tail(size_t M, size_t N, size_t K, int *splits);
  * workgroups of a smaller tile.  Returns that kernel's id (for hgemm_kernel_name), 0 if
  * the plan does not do this; hgemm_auto_plan_tail still gives the number of tiles. */
 int hgemm_auto_plan_tail_kernel(size_t M, size_t N, size_t K);
+/* 1 if the plan's main launch runs its tile's chained kernel (hgemm_mfma_chained_*), 0 if the
+ * interleaved one (hgemm_mfma_pipelined_*) or a kernel of another family. */
+int hgemm_auto_plan_chained(size_t M, size_t N, size_t K);
 const char *hgemm_kernel_name(int kernel);
 
 /* ---- workspace of hgemm_auto / hgemm_skinny.  Plans that cut K into slices keep fp32
