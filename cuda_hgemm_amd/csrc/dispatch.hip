@@ -616,10 +616,13 @@ extern "C" int hgemm_auto_plan_chained(size_t M, size_t N, size_t K) {
     const Plan p = plan_for(M, N, K);
     if (p.splits < 1) return 0;
     const size_t k_len = K / (size_t)p.splits;
+    auto workgroups = [&](size_t bm, size_t bn) {  // of the main launch
+        return (div_ceil(M, bm) * div_ceil(N, bn) - (size_t)p.tail_tiles) * (size_t)p.splits;
+    };
     switch (p.kernel) {
-        case KERNEL_BIG256: return use_chained<Big256>(PipeKernel::Auto, k_len) ? 1 : 0;
-        case KERNEL_T192: return use_chained<Tile192>(PipeKernel::Auto, k_len) ? 1 : 0;
-        case KERNEL_R256x128: return use_chained<Rect256x128>(PipeKernel::Auto, k_len) ? 1 : 0;
+        case KERNEL_BIG256: return use_chained<Big256>(PipeKernel::Auto, workgroups(256, 256), k_len) ? 1 : 0;
+        case KERNEL_T192: return use_chained<Tile192>(PipeKernel::Auto, workgroups(192, 192), k_len) ? 1 : 0;
+        case KERNEL_R256x128: return use_chained<Rect256x128>(PipeKernel::Auto, workgroups(256, 128), k_len) ? 1 : 0;
         default: return 0;
     }
 }

@@ -658,18 +658,24 @@ namespace hgemm {
 
 // Which of the two kernels runs a tile: the chained one needs a wave tile large enough that
 // one wave owns a SIMD (with two or three waves per SIMD their MFMAs interleave and nothing
-// is chained) and a K long enough to pay for its longer prologue.  Measured on an MI355X
-// against the interleaved kernel, tile by tile: ahead from K = 3072 on for 256x256, 256x128
-// and 192x192, behind everywhere for 128x128 and 64x64.
+// is chained), enough workgroups that the chip runs at its power limit (chaining saves power,
+// not issue slots) and a K long enough to pay for its longer prologue.  Measured on an MI355X
+// against the interleaved kernel, tile by tile, over grids of 64 to 1024 tiles and K from 512
+// to 8192: 256x256 ahead (1-4 %) from K = 1536 on once most CUs have a tile, 256x128 and
+// 192x192 from K = 4096 on, 128x128 and 64x64 behind everywhere.
 enum class PipeKernel { Auto, Interleaved, Chained };
 template <class Cfg>
 constexpr bool chained_available() {
     return Cfg::MI == 16 && Cfg::PTM * Cfg::PTN >= 32 && Cfg::PTN % 2 == 0 && Cfg::SA >= 3;
 }
+inline bool chained_pays(int bm, int bn, size_t workgroups, size_t k_len) {
+    if (bm == 256 && bn == 256) return (workgroups >= 192 && k_len >= 1536) || k_len >= 8192;
+    return k_len >= 4096;
+}
 template <class Cfg>
-bool use_chained(PipeKernel which, size_t k_len) {
+bool use_chained(PipeKernel which, size_t workgroups, size_t k_len) {
     if (!chained_available<Cfg>() || which == PipeKernel::Interleaved) return false;
-    return which == PipeKernel::Chained || k_len >= 3072;
+    return which == PipeKernel::Chained || chained_pays(Cfg::BM, Cfg::BN, workgroups, k_len);
 }
 
 // Launches workgroup ids [first_block, first_block + blocks) of the tile grid; tail_tiles
@@ -694,7 +700,7 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
     if (blocks < 0) blocks = tiles_m * tiles_n - first_block;
     HGEMM_CHECK(first_block >= 0 && blocks >= 1 && first_block + blocks <= tiles_m * tiles_n);
     if constexpr (chained_available<Cfg>()) {
-        if (use_chained<Cfg>(which, K / (size_t)splits)) {
+        if (use_chained<Cfg>(which, (size_t)blocks * (size_t)splits, K / (size_t)splits)) {
             hgemm_chained_kernel<Cfg, SPLIT, EDGE><<<dim3(blocks, splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
                 reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
                 partial, (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, first_block, tail_tiles,

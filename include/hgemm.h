@@ -97,7 +97,7 @@ HGEMM_FUNC(hgemm_mfma_pipelined_64x64);
  * its two MFMAs back to back (the matrix pipe forwards the running sum instead of going
  * through the register file: less power, hence more clock) and with the accumulators in
  * registers the compiler never sees.  The top of the ladder; hgemm_auto runs these on large
- * shapes with K >= 3072.  Same shape needs as the pipelined entry points above. */
+ * grids with long K (256x256: from K = 1536 once most CUs have a tile; the others from 4096).  Same shape needs as the pipelined entry points above. */
 HGEMM_FUNC(hgemm_mfma_chained_256x256);
 HGEMM_FUNC(hgemm_mfma_chained_256x128);
 HGEMM_FUNC(hgemm_mfma_chained_192x192);

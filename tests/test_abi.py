@@ -92,8 +92,10 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
         p = plan(n, n, n)
         assert p["kernel"] != "scalar fallback" and p["splits"] >= 1, (n, p)
     assert plan(8192, 8192, 8192)["kernel"].startswith("pipelined 256x256") and plan(8192, 8192, 8192)["chained"]
-    assert not plan(4096, 4096, 2048)["chained"] and not plan(1024, 1024, 8192)["chained"]   # short K; small tile
-    assert plan(3072, 3072, 3072)["kernel"].startswith("pipelined 192x192") and plan(3072, 3072, 3072)["chained"]
+    assert plan(4096, 4096, 2048)["chained"] and not plan(4096, 4096, 1024)["chained"]       # 256 tiles: from K = 1536
+    assert not plan(2048, 2048, 4096)["chained"] and not plan(1024, 1024, 8192)["chained"]   # few tiles; small tile
+    assert plan(3072, 3072, 3072)["kernel"].startswith("pipelined 192x192") and not plan(3072, 3072, 3072)["chained"]
+    assert plan(3072, 3072, 4096)["kernel"].startswith("pipelined 192x192") and plan(3072, 3072, 4096)["chained"]
     for shape in ((4096, 14336, 4096), (4096, 4096, 14336)):
         assert plan(*shape)["kernel"].startswith("pipelined"), shape
     for m in (1, 8, 16, 64, 128):
