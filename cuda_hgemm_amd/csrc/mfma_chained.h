@@ -141,7 +141,10 @@ __global__ void __launch_bounds__(Cfg::THREADS)
 
     int tile_m, tile_n;
     if (subdiv == 0) {
-        tile_of_block<Cfg>(first_block + (int)blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+        // positions [first_block, first_block + gridDim.x) of the tile order, contiguous per XCD; a launch
+        // whose partial sums are indexed by blockIdx.x (tail_tiles > 0) keeps the plain order the reduction uses
+        const int pos = tail_tiles > 0 ? (int)blockIdx.x : xcd_contiguous((int)blockIdx.x, (int)gridDim.x);
+        tile_of_block<Cfg>(first_block + pos, tiles_m, tiles_n, tile_m, tile_n);
     } else {
         // tiles_m x tiles_n is the grid of a larger tile that this one divides sub_m x sub_n times;
         // consecutive workgroups take the parts of workgroup id first_block + blockIdx.x / parts

@@ -118,16 +118,20 @@ __device__ __forceinline__ int swizzle_of_row(int row) {
     return ((line & 7) ^ ((line >> 3) & 1)) & (Cfg::CPR - 1);
 }
 
-// Tile owned by workgroup `bid`.  Workgroups are dealt round-robin to the 8 XCDs (each
-// with its own L2), so the id is first regrouped so that every XCD walks a contiguous
-// range of tiles, then tiles are ordered in GROUP_N-wide strips walked down M: the
-// workgroups resident together on one XCD share a few A and B panels in that L2.
+// Workgroups of a launch are dealt round-robin to the 8 XCDs, each with its own L2: workgroup
+// b runs on XCD b % 8.  This maps b to a position in [0, count) such that every XCD walks a
+// contiguous range of positions (XCD x gets count / 8 of them, the first count % 8 XCDs one
+// more), so that the workgroups resident together on one XCD are neighbours in tile order.
+__device__ __forceinline__ int xcd_contiguous(int b, int count) {
+    const int x = b & 7, q = count >> 3, r = count & 7;
+    return x * q + (x < r ? x : r) + (b >> 3);
+}
+
+// Tile at position `lin` of the tile order: GROUP_N-wide strips walked down M, so that
+// neighbouring positions share a few A and B panels (in the L2 of the XCD they run on).
 // (Counterpart of the reference's 16-tile strips, src/mma/mma_base.cu:51-53.)
 template <class Cfg>
-__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
-    const int total = tiles_m * tiles_n;
-    int lin = bid;
-    if ((total & 7) == 0) lin = (bid & 7) * (total >> 3) + (bid >> 3);
+__device__ __forceinline__ void tile_of_block(int lin, int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
     const int strip_tiles = Cfg::GROUP_N * tiles_m;
     const int strip = lin / strip_tiles;
     const int within = lin - strip * strip_tiles;
@@ -197,7 +201,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
 
     int tile_m, tile_n;
-    tile_of_block<Cfg>(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_block<Cfg>(xcd_contiguous((int)blockIdx.x, (int)gridDim.x), tiles_m, tiles_n, tile_m, tile_n);
 
     const half_t *Ag = A + (size_t)tile_m * BM * K;
     const half_t *Bg = B + (size_t)tile_n * BN * K;

@@ -48,7 +48,7 @@ __global__ void __launch_bounds__(256) mix(const half_t *A, const half_t *B, flo
     constexpr int MODE = (MODE_ >= 5) ? 1 : MODE_;
     constexpr int CHAIN = MODE_ == 6 ? 2 : (MODE_ == 7 ? 4 : 1);
     for (int bid = blockIdx.x; bid < tiles_m * tiles_n; bid += gridDim.x) {
-    tile_of_block<RasterCfg>(bid, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_block<RasterCfg>(xcd_contiguous(bid, tiles_m * tiles_n), tiles_m, tiles_n, tile_m, tile_n);
     uint32_t s = tid * 7919u + blockIdx.x * 104729u + 1;
     half8 a[8], b[8];
     for (int i = 0; i < 8; ++i) { a[i] = rnd8(s); b[i] = rnd8(s); }
