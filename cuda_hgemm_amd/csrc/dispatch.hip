@@ -131,7 +131,7 @@ using Split128x64 = SkinnyConfig<128, 64, 2, 2, 4>;
 using Split128x128 = SkinnyConfig<128, 128, 2, 2, 4>;
 
 // 256x256x64 tile on v_mfma_f32_16x16x32_f16, two B buffers and three A buffers (all 160 KB of LDS)
-using Big256 = PipeConfig<256, 256, 64, 2, 2, 2, 16, 8, 0, 1>;
+using Big256 = PipeConfig<256, 256, 64, 2, 2, 2, 16, 0, 1>;
 using Mid128 = PipeConfig<128, 128, 64, 2, 2, 5, 16>;
 using Mid128S4 = PipeConfig<128, 128, 64, 2, 2, 4, 16>;
 using Small64 = PipeConfig<64, 64, 64, 1, 1, 3, 16>;

@@ -140,22 +140,26 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
 
     int tile_m, tile_n;
+    const bool blocked = blocked_order(N, K);  // the same in every launch that works on this problem
+    // this workgroup's slot among the launch's gridDim.x: slots are dealt so that the workgroups an XCD runs
+    // together are neighbours in the tile order
+    const int slot = slot_of_workgroup(blocked, (int)blockIdx.x, (int)gridDim.x);
     if (subdiv == 0) {
-        // positions [first_block, first_block + gridDim.x) of the tile order, contiguous per XCD; a launch
-        // whose partial sums are indexed by blockIdx.x (tail_tiles > 0) keeps the plain order the reduction uses
-        const int pos = tail_tiles > 0 ? (int)blockIdx.x : xcd_contiguous((int)blockIdx.x, (int)gridDim.x);
-        tile_of_block<Cfg>(first_block + pos, tiles_m, tiles_n, tile_m, tile_n);
+        // the launch covers positions [first_block, first_block + gridDim.x) of the tile order
+        tile_of_position(blocked, first_block + slot, tiles_m, tiles_n, tile_m, tile_n);
     } else {
         // tiles_m x tiles_n is the grid of a larger tile that this one divides sub_m x sub_n times;
-        // consecutive workgroups take the parts of workgroup id first_block + blockIdx.x / parts
+        // consecutive slots take the parts of the tile at position first_block + slot / parts
         const int sub_m = subdiv >> 8, sub_n = subdiv & 255, parts = sub_m * sub_n;
-        const int part = (int)blockIdx.x % parts;
+        const int part = slot % parts;
         int parent_m, parent_n;
-        tile_of_block<Cfg>(first_block + (int)blockIdx.x / parts, tiles_m, tiles_n, parent_m, parent_n);
+        tile_of_position(blocked, first_block + slot / parts, tiles_m, tiles_n, parent_m, parent_n);
         tile_m = parent_m * sub_m + part / sub_n;
         tile_n = parent_n * sub_n + part % sub_n;
         if (tile_m * BM >= M || tile_n * BN >= N) return;  // a part wholly outside the matrix (whole workgroup)
     }
+    tile_m = __builtin_amdgcn_readfirstlane(tile_m);  // wave-uniform by construction: keep them in SGPRs
+    tile_n = __builtin_amdgcn_readfirstlane(tile_n);
     const int num_k = k_len / BK;
     const int k_begin = SPLIT ? (int)blockIdx.y * k_len : 0;
 
@@ -441,11 +445,17 @@ __global__ void __launch_bounds__(Cfg::THREADS)
                 // The sources of the next window, a few scalar instructions at a time in slots that
                 // host nothing else (block 1: no copy of this window's start is issued before the barrier).
                 if constexpr (!FINAL && j == 1 && sl == 3) {
-                    a_off_far = a_off_far + BK * 2 < last_off ? a_off_far + BK * 2 : last_off;
+                    if constexpr (Cfg::DBG_MODE == 2)  // probe build: the same two chunks over and over (L2 hits)
+                        a_off_far = a_off_far == 0 ? BK * 2 : 0;
+                    else
+                        a_off_far = a_off_far + BK * 2 < last_off ? a_off_far + BK * 2 : last_off;
                     a_post = a_base + a_off_far;
                 }
                 if constexpr (!FINAL && j == 1 && sl == 5) {
-                    b_off_far = b_off_far + BK * 2 < last_off ? b_off_far + BK * 2 : last_off;
+                    if constexpr (Cfg::DBG_MODE == 2)
+                        b_off_far = b_off_far == 0 ? BK * 2 : 0;
+                    else
+                        b_off_far = b_off_far + BK * 2 < last_off ? b_off_far + BK * 2 : last_off;
                     b_post = b_base + b_off_far;
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -526,7 +536,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         // a lane holds four consecutive n of row m = lane % 16 of each 16x16 tile: 16 bytes of fp32
         const int row = tile_m * BM + wm * Cfg::WM + lane_late % MI, col = tile_n * BN + wn * Cfg::WN + (lane_late / MI) * 4;
         if (tail_tiles > 0) {  // compact: whole tiles, nothing to guard
-            float *dst = partial + ((size_t)blockIdx.y * tail_tiles + blockIdx.x) * (BM * BN) +
+            float *dst = partial + ((size_t)blockIdx.y * tail_tiles + slot) * (BM * BN) +
                          (wm * Cfg::WM + lane_late % MI) * BN + wn * Cfg::WN + (lane_late / MI) * 4;
             static_for<TM>([&](auto i_c) {
                 static_for<TN>([&](auto j_c) {

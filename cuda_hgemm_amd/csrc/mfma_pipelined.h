@@ -21,10 +21,10 @@
 
 namespace hgemm {
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int MI_ = 16, int GROUP_N_ = 8,
-          int DBG_ = 0, int EXTRA_A_ = 0>
-struct PipeConfig : TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true, GROUP_N_> {
-    using Base = TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true, GROUP_N_>;
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int MI_ = 16, int DBG_ = 0,
+          int EXTRA_A_ = 0>
+struct PipeConfig : TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true> {
+    using Base = TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true>;
     // MFMA shape: 32 -> v_mfma_f32_32x32x16_f16, 16 -> v_mfma_f32_16x16x32_f16.  Both move
     // the same bytes from LDS per flop (that depends on the wave tile only); the 16x16x32
     // form reads and writes half as many accumulator registers per flop and sustains a
@@ -254,22 +254,26 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
 
     int tile_m, tile_n;
+    const bool blocked = blocked_order(N, K);  // the same in every launch that works on this problem
+    // this workgroup's slot among the launch's gridDim.x: slots are dealt so that the workgroups an XCD runs
+    // together are neighbours in the tile order
+    const int slot = slot_of_workgroup(blocked, (int)blockIdx.x, (int)gridDim.x);
     if (subdiv == 0) {
-        // positions [first_block, first_block + gridDim.x) of the tile order, contiguous per XCD; a launch
-        // whose partial sums are indexed by blockIdx.x (tail_tiles > 0) keeps the plain order the reduction uses
-        const int pos = tail_tiles > 0 ? (int)blockIdx.x : xcd_contiguous((int)blockIdx.x, (int)gridDim.x);
-        tile_of_block<Cfg>(first_block + pos, tiles_m, tiles_n, tile_m, tile_n);
+        // the launch covers positions [first_block, first_block + gridDim.x) of the tile order
+        tile_of_position(blocked, first_block + slot, tiles_m, tiles_n, tile_m, tile_n);
     } else {
         // tiles_m x tiles_n is the grid of a larger tile that this one divides sub_m x sub_n times;
-        // consecutive workgroups take the parts of workgroup id first_block + blockIdx.x / parts
+        // consecutive slots take the parts of the tile at position first_block + slot / parts
         const int sub_m = subdiv >> 8, sub_n = subdiv & 255, parts = sub_m * sub_n;
-        const int part = (int)blockIdx.x % parts;
+        const int part = slot % parts;
         int parent_m, parent_n;
-        tile_of_block<Cfg>(first_block + (int)blockIdx.x / parts, tiles_m, tiles_n, parent_m, parent_n);
+        tile_of_position(blocked, first_block + slot / parts, tiles_m, tiles_n, parent_m, parent_n);
         tile_m = parent_m * sub_m + part / sub_n;
         tile_n = parent_n * sub_n + part % sub_n;
         if (tile_m * BM >= M || tile_n * BN >= N) return;  // a part wholly outside the matrix (whole workgroup)
     }
+    tile_m = __builtin_amdgcn_readfirstlane(tile_m);  // wave-uniform by construction: keep them in SGPRs
+    tile_n = __builtin_amdgcn_readfirstlane(tile_n);
     const int num_k = k_len / BK;
     const int k_begin = SPLIT ? (int)blockIdx.y * k_len : 0;
 
@@ -574,7 +578,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         // a lane holds four consecutive n of row m = lane % 16 of each 16x16 tile: 16 bytes of fp32
         const int row = tile_m * BM + wm * Cfg::WM + lane % MI, col = tile_n * BN + wn * Cfg::WN + (lane / MI) * 4;
         if (tail_tiles > 0) {  // compact: whole tiles, nothing to guard
-            float *dst = partial + ((size_t)blockIdx.y * tail_tiles + blockIdx.x) * (BM * BN) +
+            float *dst = partial + ((size_t)blockIdx.y * tail_tiles + slot) * (BM * BN) +
                          (wm * Cfg::WM + lane % MI) * BN + wn * Cfg::WN + (lane / MI) * 4;
             static_for<TM>([&](auto i_c) {
                 static_for<TN>([&](auto j_c) {
@@ -625,12 +629,12 @@ bool pipelined_supports_edges(size_t M, size_t N, size_t K) {
 // slices added in order; rows and 8-column pieces outside the matrix are skipped.
 template <class Cfg>
 __global__ void __launch_bounds__(256)
-    tail_reduce_kernel(const float *__restrict__ partial, half_t *__restrict__ C, int M, int N, int tiles_m, int tiles_n,
-                       int first_block, int tail_tiles, int splits) {
+    tail_reduce_kernel(const float *__restrict__ partial, half_t *__restrict__ C, int M, int N, int K, int tiles_m,
+                       int tiles_n, int first_block, int tail_tiles, int splits) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, PIECES = BM * BN / 8;
     const int t = blockIdx.y;
     int tile_m, tile_n;
-    tile_of_block<Cfg>(first_block + t, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_position(blocked_order(N, K), first_block + t, tiles_m, tiles_n, tile_m, tile_n);
     const size_t slice_stride = (size_t)tail_tiles * (BM * BN);
     for (int piece = blockIdx.x * blockDim.x + threadIdx.x; piece < PIECES; piece += gridDim.x * blockDim.x) {
         const int r = piece / (BN / 8), c = (piece % (BN / 8)) * 8;
@@ -744,7 +748,7 @@ void launch_pipelined_with_tail(const void *A, const void *B, void *C, float *pa
     }
     constexpr int PIECES = Cfg::BM * Cfg::BN / 8;
     tail_reduce_kernel<Cfg><<<dim3(PIECES / 256 > 8 ? 8 : (PIECES + 255) / 256, tail_tiles), dim3(256), 0, nullptr>>>(
-        partial, reinterpret_cast<half_t *>(C), (int)M, (int)N, tiles_m, tiles_n, head, tail_tiles, tail_splits);
+        partial, reinterpret_cast<half_t *>(C), (int)M, (int)N, (int)K, tiles_m, tiles_n, head, tail_tiles, tail_splits);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 
@@ -786,8 +790,8 @@ void launch_pipelined_split(const void *A, const void *B, float *partial, size_t
 template <class Parent, class Child>
 void launch_pipelined_with_subtiles(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, int tail_tiles,
                                     const char *name) {
-    static_assert(Parent::BM % Child::BM == 0 && Parent::BN % Child::BN == 0 && Parent::GROUP_N == Child::GROUP_N,
-                  "the child tile must divide the parent tile and share its rasterisation");
+    static_assert(Parent::BM % Child::BM == 0 && Parent::BN % Child::BN == 0,
+                  "the child tile must divide the parent tile");
     check_operands(A, B, C, M, N, K);
     constexpr int sub_m = Parent::BM / Child::BM, sub_n = Parent::BN / Child::BN;
     const int tiles_m = (int)div_ceil(M, (size_t)Parent::BM), tiles_n = (int)div_ceil(N, (size_t)Parent::BN);

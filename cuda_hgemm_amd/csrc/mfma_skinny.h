@@ -20,7 +20,7 @@
 namespace hgemm {
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_>
-struct SkinnyConfig : TileConfig<BM_, BN_, 64, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true, 1> {};
+struct SkinnyConfig : TileConfig<BM_, BN_, 64, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true> {};
 
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS)

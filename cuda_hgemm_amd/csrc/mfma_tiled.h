@@ -23,6 +23,7 @@
 #include <stdint.h>
 
 #include "common.h"
+#include "tile_order.h"
 
 namespace hgemm {
 
@@ -38,13 +39,12 @@ enum { LOAD_REG = 0, LOAD_DMA = 1 };
 enum { LDS_LINEAR = 0, LDS_PADDED = 1, LDS_SWIZZLE = 2 };
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int LOADER_, int LAYOUT_,
-          bool FRAG_PREFETCH_, int GROUP_N_ = 8>
+          bool FRAG_PREFETCH_>
 struct TileConfig {
     static constexpr int BM = BM_, BN = BN_, BK = BK_;
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int STAGES = STAGES_, LOADER = LOADER_, LAYOUT = LAYOUT_;
     static constexpr bool FRAG_PREFETCH = FRAG_PREFETCH_;
-    static constexpr int GROUP_N = GROUP_N_;  // rasterisation strip width in tiles
 
     static constexpr int WAVES = WAVES_M * WAVES_N;
     static constexpr int THREADS = WAVES * 64;
@@ -118,29 +118,6 @@ __device__ __forceinline__ int swizzle_of_row(int row) {
     return ((line & 7) ^ ((line >> 3) & 1)) & (Cfg::CPR - 1);
 }
 
-// Workgroups of a launch are dealt round-robin to the 8 XCDs, each with its own L2: workgroup
-// b runs on XCD b % 8.  This maps b to a position in [0, count) such that every XCD walks a
-// contiguous range of positions (XCD x gets count / 8 of them, the first count % 8 XCDs one
-// more), so that the workgroups resident together on one XCD are neighbours in tile order.
-__device__ __forceinline__ int xcd_contiguous(int b, int count) {
-    const int x = b & 7, q = count >> 3, r = count & 7;
-    return x * q + (x < r ? x : r) + (b >> 3);
-}
-
-// Tile at position `lin` of the tile order: GROUP_N-wide strips walked down M, so that
-// neighbouring positions share a few A and B panels (in the L2 of the XCD they run on).
-// (Counterpart of the reference's 16-tile strips, src/mma/mma_base.cu:51-53.)
-template <class Cfg>
-__device__ __forceinline__ void tile_of_block(int lin, int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
-    const int strip_tiles = Cfg::GROUP_N * tiles_m;
-    const int strip = lin / strip_tiles;
-    const int within = lin - strip * strip_tiles;
-    const int n_first = strip * Cfg::GROUP_N;
-    const int width = (tiles_n - n_first) < Cfg::GROUP_N ? (tiles_n - n_first) : Cfg::GROUP_N;
-    tile_m = within / width;
-    tile_n = n_first + within % width;
-}
-
 // Epilogue shared by the tiled kernels: accumulators -> fp16 -> C, staged through LDS.
 // A lane of the (operand-swapped) accumulator holds four consecutive n of one row; stored
 // straight to global memory that is 16 useful bytes per 32 rows per instruction, i.e. a
@@ -201,7 +178,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
 
     int tile_m, tile_n;
-    tile_of_block<Cfg>(xcd_contiguous((int)blockIdx.x, (int)gridDim.x), tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup(blocked_order(N, K), 0, (int)blockIdx.x, (int)gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
 
     const half_t *Ag = A + (size_t)tile_m * BM * K;
     const half_t *Bg = B + (size_t)tile_n * BN * K;

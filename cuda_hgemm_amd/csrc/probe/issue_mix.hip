@@ -34,7 +34,6 @@ __device__ inline half8 rnd8(uint32_t &s) {
     for (int i = 0; i < 8; ++i) { s = s * 1664525u + 1013904223u; v[i] = (_Float16)(((int)(s >> 8) % 2001 - 1000) * 0.001f); }
     return v;
 }
-struct RasterCfg { static constexpr int GROUP_N = 8; };
 
 // ---- part 1: the loop's instruction mix (modes in the header of this file)
 template <int MODE_>
@@ -48,7 +47,8 @@ __global__ void __launch_bounds__(256) mix(const half_t *A, const half_t *B, flo
     constexpr int MODE = (MODE_ >= 5) ? 1 : MODE_;
     constexpr int CHAIN = MODE_ == 6 ? 2 : (MODE_ == 7 ? 4 : 1);
     for (int bid = blockIdx.x; bid < tiles_m * tiles_n; bid += gridDim.x) {
-    tile_of_block<RasterCfg>(xcd_contiguous(bid, tiles_m * tiles_n), tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup(false, 0, bid, tiles_m * tiles_n, tiles_m, tiles_n, tile_m, tile_n);
+    tile_m = __builtin_amdgcn_readfirstlane(tile_m); tile_n = __builtin_amdgcn_readfirstlane(tile_n);
     uint32_t s = tid * 7919u + blockIdx.x * 104729u + 1;
     half8 a[8], b[8];
     for (int i = 0; i < 8; ++i) { a[i] = rnd8(s); b[i] = rnd8(s); }

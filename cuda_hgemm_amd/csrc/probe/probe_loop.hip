@@ -21,7 +21,7 @@ namespace {
 
 // DBG 8: timestamps only; + 1: no copies; + 2: copies from a fixed K offset; + 4: no operand reads
 template <int DBG>
-using ProbeConfig = PipeConfig<256, 256, 64, 2, 2, 2, 16, 8, DBG, 1>;
+using ProbeConfig = PipeConfig<256, 256, 64, 2, 2, 2, 16, DBG, 1>;
 
 template <int DBG, PipeKernel WHICH = PipeKernel::Interleaved>
 void run_probe(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, size_t launches, double *out) {
