@@ -140,7 +140,8 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
 
     int tile_m, tile_n;
-    const bool blocked = blocked_order(N, K);  // the same in every launch that works on this problem
+    // the same in every launch that works on this problem (probe builds can force either order)
+    const bool blocked = (Cfg::DBG & 16) ? false : ((Cfg::DBG & 32) ? true : blocked_order(N, K));
     // this workgroup's slot among the launch's gridDim.x: slots are dealt so that the workgroups an XCD runs
     // together are neighbours in the tile order
     const int slot = slot_of_workgroup(blocked, (int)blockIdx.x, (int)gridDim.x);

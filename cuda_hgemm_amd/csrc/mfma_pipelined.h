@@ -35,8 +35,9 @@ struct PipeConfig : TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_
     static constexpr int PKSTEPS = BK_ / PKSTEP;
     static constexpr int CPS = PKSTEP / 8;                          // 16-byte chunks per row per step
     // Timing experiments only (the library instantiates DBG = 0, which compiles none of it):
-    // 1 = no copies in the loop, 2 = copies from a fixed K offset, 4 = no operand reads in
-    // the loop; any non-zero value also records per-workgroup timestamps into `probe_out`.
+    // low three bits: 1 = no copies in the loop, 2 = copies from a fixed K offset, 4 = no operand
+    // reads in the loop; + 16 / + 32 = strip / block tile order regardless of the problem; any
+    // non-zero value also records per-workgroup timestamps into `probe_out`.
     static constexpr int DBG = DBG_;
     static constexpr int DBG_MODE = DBG_ & 7;
     static constexpr bool TIMESTAMPS = DBG_ != 0;
@@ -254,7 +255,8 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
 
     int tile_m, tile_n;
-    const bool blocked = blocked_order(N, K);  // the same in every launch that works on this problem
+    // the same in every launch that works on this problem (probe builds can force either order)
+    const bool blocked = (Cfg::DBG & 16) ? false : ((Cfg::DBG & 32) ? true : blocked_order(N, K));
     // this workgroup's slot among the launch's gridDim.x: slots are dealt so that the workgroups an XCD runs
     // together are neighbours in the tile order
     const int slot = slot_of_workgroup(blocked, (int)blockIdx.x, (int)gridDim.x);

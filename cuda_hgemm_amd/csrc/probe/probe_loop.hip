@@ -19,7 +19,8 @@
 namespace hgemm {
 namespace {
 
-// DBG 8: timestamps only; + 1: no copies; + 2: copies from a fixed K offset; + 4: no operand reads
+// DBG 8: timestamps only; + 1: no copies; + 2: copies from a fixed K offset; + 4: no operand reads;
+// + 16 / + 32: tiles in the strip / block order whatever the size of B
 template <int DBG>
 using ProbeConfig = PipeConfig<256, 256, 64, 2, 2, 2, 16, DBG, 1>;
 
@@ -92,12 +93,14 @@ int main(int argc, char *argv[]) {
     const FillSpec uniform;
     Matrix A(M, K, "Matrix A", flags.u64("seed"), 1, uniform), B(K, N, "Matrix B", flags.u64("seed"), 2, uniform);
     Matrix C(M, N, "Matrix C", flags.u64("seed"), 3, FillSpec{Fill::Zero, 0.f, 0.f});
-    static const char *names[8] = {"interleaved kernel", "interleaved, copies always from the same two chunks (all L2 hits)",
+    static const char *names[10] = {"interleaved kernel", "interleaved, copies always from the same two chunks (all L2 hits)",
                                    "interleaved, loop without copies", "interleaved, loop without copies and operand reads",
                                    "chained kernel", "chained, copies always from the same two chunks (all L2 hits)",
-                                   "chained, loop without copies", "chained, loop without copies and operand reads"};
+                                   "chained, loop without copies", "chained, loop without copies and operand reads",
+                                   "chained, tiles in strips (the order for a B of at most 144 MiB)",
+                                   "chained, tiles in 16 x 16 blocks per round (the order for a larger B)"};
     constexpr PipeKernel CH = PipeKernel::Chained;
-    for (int mode = 0; mode < 8; ++mode) {
+    for (int mode = 0; mode < 10; ++mode) {
         double r[8];
         const uint16_t *a = A.getDevPtr(), *b = B.getDevPtr();
         uint16_t *c = C.getDevPtr();
@@ -109,7 +112,9 @@ int main(int argc, char *argv[]) {
             case 4: run_probe<8, CH>(a, b, c, M, N, K, launches, r); break;
             case 5: run_probe<8 + 2, CH>(a, b, c, M, N, K, launches, r); break;
             case 6: run_probe<8 + 1, CH>(a, b, c, M, N, K, launches, r); break;
-            default: run_probe<8 + 4, CH>(a, b, c, M, N, K, launches, r); break;
+            case 7: run_probe<8 + 4, CH>(a, b, c, M, N, K, launches, r); break;
+            case 8: run_probe<8 + 16, CH>(a, b, c, M, N, K, launches, r); break;
+            default: run_probe<8 + 32, CH>(a, b, c, M, N, K, launches, r); break;
         }
         HLOG("Probe %s: %zu launches avg %.4f ms, traced launch %.4f ms (%.1f TFLOPS); per workgroup: prologue "
              "%.2f us, loop %.2f us, epilogue %.2f us; loop %.0f shader cycles at %.3f GHz, MFMA issue %.1f%%",
