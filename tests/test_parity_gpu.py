@@ -289,6 +289,29 @@ def test_auto_last_round_of_a_large_grid(oracle, hgemm_lib, gpu, shape, mode):
     assert np.array_equal(got[M - 8:], oracle.hgemm_rows(At, Bt, M - 8, 8))
 
 
+@pytest.mark.parametrize("variant,shape", [
+    ("hgemm_auto", (520, 9480, 8192)),                    # 3 x 38 tiles of 256: clipped blocks, ragged M and N
+    ("hgemm_auto", (4352, 9472, 8192)),                   # 17 x 37 tiles: whole rounds plus a last, separately launched one
+    ("hgemm_mfma_chained_256x256", (2304, 9472, 8192)),   # 9 x 37 tiles in one launch
+    ("hgemm_mfma_pipelined_256x256", (2304, 9472, 8192)),
+    ("hgemm_mfma_pipelined_128x128", (648, 9480, 8192)),  # 6 x 75 tiles of 128, three workgroups per round and XCD
+    ("hgemm_mfma_async_stage4", (512, 9472, 8192)),       # the ladder's 256 x 128 tiles: 2 x 74
+])
+def test_block_tile_order(oracle, hgemm_lib, gpu, variant, shape):
+    """A B of more than 144 MiB switches the tuned kernels (and the ladder) to the order that
+    deals 16 x 16 blocks of tiles per round: every tile must still be computed exactly once,
+    whatever the grid and however the launch is cut.  C starts as NaN, so a tile nobody
+    computes shows; ternary inputs make complete rows exact, rows taken from every row of tiles."""
+    M, N, K = shape
+    assert N * K > 72 << 20
+    At, Bt = oracle.fill((M, K), 43, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 43, 2, oracle.TERNARY, 0, 1)
+    first, second = _run(hgemm_lib, variant, At, Bt, gpu, repeat=2)
+    assert not np.any((first & 0x7C00) == 0x7C00), "outputs left unwritten or non-finite"
+    assert np.array_equal(first, second)
+    rows = np.unique(np.concatenate([np.arange(m0, m0 + 4) for m0 in list(range(0, M - 8, 61)) + [M - 4]]))
+    assert np.array_equal(first[rows], oracle.hgemm(np.ascontiguousarray(At[rows]), Bt))
+
+
 @pytest.mark.parametrize("N", [4096, 28672])
 @pytest.mark.parametrize("M", [1, 8, 16, 64, 128])
 def test_decode_shapes(oracle, hgemm_lib, gpu, M, N):
