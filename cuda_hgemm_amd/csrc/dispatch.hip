@@ -137,6 +137,9 @@ using Mid128S4 = PipeConfig<128, 128, 64, 2, 2, 4, 16>;
 using Small64 = PipeConfig<64, 64, 64, 1, 1, 3, 16>;
 using Tile192 = PipeConfig<192, 192, 64, 2, 2, 3, 16>;
 using Rect256x128 = PipeConfig<256, 128, 64, 2, 2, 3, 16>;
+// 64x64x64 on four waves (one 32x32 MFMA tile each) with the ladder's kernel: a small tile whose chunk takes a quarter
+// of the one-wave tile's matrix-pipe time; for grids that give a CU at most one tile
+using Small64W4 = TileConfig<64, 64, 64, 2, 2, 3, LOAD_DMA, LDS_SWIZZLE, true>;
 
 // Pipelined kernel with K cut into `splits` slices: fp32 partial sums per slice, then the
 // ordered reduction (the same one the small-M kernel uses), so the result is bit-identical
@@ -192,6 +195,9 @@ constexpr Candidate CANDIDATES[] = {
     {KERNEL_R256x128, 256, 128, 1, 3, 4.25, 0.476, 0.856},
     {KERNEL_MID128, 128, 128, 1, 5, 3.17, 0.266, 0.510},
     {KERNEL_SMALL64, 64, 64, 3, 3, 1.39, 0.294, 0.585},
+    // whole tiles only, no K slices; fitted on 16 to 256 tiles (256^3 ... 1024^3, K to 4096), where it is 13-22 % ahead of
+    // the one-wave tile; modelled at one workgroup per CU, which keeps it out of larger grids (where it is behind)
+    {KERNEL_SMALL64_W4, 64, 64, 1, 3, 1.94, 0.216, 0.246},
 };
 // launch; reduction kernel: fixed + per slice + fp32 partials written and read back
 constexpr double LAUNCH_US = 0.16, REDUCE_US = 3.90, REDUCE_SLICE_US = 0.10, REDUCE_BYTES_PER_US = 7040e3;
@@ -301,7 +307,13 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     double best = 0.0;
     for (const Candidate &c : CANDIDATES) {
         if (N % 8) break;
+        const bool whole_tiles_only = c.kernel == KERNEL_SMALL64_W4;
+        if (whole_tiles_only && (M % c.bm || N % c.bn)) continue;
         for (int s = 1; s <= 32; s *= 2) {
+            if (whole_tiles_only && s > 1) break;
+            // whole 64x64 tiles, at most one per CU, no K slices: the four-wave tile is ahead of the one-wave tile on
+            // every such grid that was measured (the model, fitted on larger grids, flatters the one-wave tile there)
+            if (c.kernel == KERNEL_SMALL64 && s == 1 && M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) <= cus) continue;
             if (K % ((size_t)s * 64) || K / s < (size_t)64 * c.stages) break;
             if (s > 1 && (size_t)s * slice_bytes > limits.partial_bytes) break;
             const double t = predict_us(c, M, N, K, s, cus);
@@ -319,7 +331,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
         // a grid of whole rounds plus a few workgroups: run those few in K slices
         const size_t wgs = div_ceil(M, (size_t)c.bm) * div_ceil(N, (size_t)c.bn), slots = cus * (size_t)c.per_cu;
         const size_t rem = wgs % slots;
-        if (wgs > slots && rem > 0) {
+        if (wgs > slots && rem > 0 && !whole_tiles_only) {
             for (int ts = 2; ts <= 16; ts *= 2) {
                 if (K % ((size_t)ts * 64) || K / ts < (size_t)64 * c.stages || rem * ts > slots) break;
                 if ((size_t)ts * rem * c.bm * c.bn * sizeof(float) > limits.partial_bytes) break;
@@ -337,7 +349,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
             }
             if (c.kernel == KERNEL_BIG256) {  // ... or on smaller tiles that divide this one
                 for (const Candidate &small : CANDIDATES) {
-                    if (small.kernel == KERNEL_BIG256 || c.bm % small.bm || c.bn % small.bn) continue;
+                    if (small.kernel == KERNEL_BIG256 || small.kernel == KERNEL_SMALL64_W4 || c.bm % small.bm || c.bn % small.bn) continue;
                     if (K < (size_t)64 * small.stages) continue;
                     const double t = predict_subtile_us(c, small, M, N, K, cus);
                     if (p.kernel != KERNEL_NONE && t < best) {
@@ -453,6 +465,7 @@ void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, 
         case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128_S4: launch_pipelined<Mid128S4>(A, B, C, M, N, K, "hgemm_auto"); break;
         case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p, ws); break;
+        case KERNEL_SMALL64_W4: launch_tiled<Small64W4>(A, B, C, M, N, K, "hgemm_auto"); break;
         case KERNEL_SPLIT_32x64: launch_splitk<Split32x64>(A, B, C, M, N, K, p.splits, ws); break;
         case KERNEL_SPLIT_64x64: launch_splitk<Split64x64>(A, B, C, M, N, K, p.splits, ws); break;
         case KERNEL_SPLIT_64x128: launch_splitk<Split64x128>(A, B, C, M, N, K, p.splits, ws); break;
@@ -632,6 +645,7 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
         case KERNEL_MID128: return "pipelined 128x128x64, 4 waves, 5-stage ring";
         case KERNEL_MID128_S4: return "pipelined 128x128x64, 4 waves, 4-stage ring";
         case KERNEL_SMALL64: return "pipelined 64x64x64, 1 wave, 3-stage ring";
+        case KERNEL_SMALL64_W4: return "tiled 64x64x64, 4 waves of 32x32, 3-stage ring";
         case KERNEL_T192: return "pipelined 192x192x64, 4 waves, 3-stage ring";
         case KERNEL_R256x128: return "pipelined 256x128x64, 4 waves, 3-stage ring";
         case KERNEL_SPLIT_32x64: return "split-K 32x64x64, 2 waves, 4-stage ring";

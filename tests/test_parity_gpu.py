@@ -245,12 +245,14 @@ def test_auto_16384_sampled_rows(oracle, hgemm_lib, gpu):
 
 @pytest.mark.parametrize("shape,tile,split", [
     ((3072, 3072, 256), "192x192x64", False), ((2560, 2560, 256), "256x128x64", False),
-    ((256, 256, 8192), "64x64x64", True), ((1024, 1024, 4096), "128x128x64", True),
+    ((256, 256, 8192), "64x64x64", True), ((1024, 1024, 8192), "128x128x64", True),
+    ((1024, 1024, 4096), "tiled 64x64x64", False), ((512, 768, 640), "tiled 64x64x64", False), ((192, 192, 192), "tiled 64x64x64", False),
     ((512, 512, 8192), "64x64x64", True), ((1536, 1536, 16384), "192x192x64", True),
     ((2048, 2048, 16384), "256x256x64", True)])
 def test_auto_every_tile_with_and_without_k_slices(oracle, hgemm_lib, gpu, shape, tile, split):
     """Shapes chosen so the dispatcher's cost model lands on each pipelined tile, alone and
-    with K cut into slices (fp32 partial sums + ordered reduction)."""
+    with K cut into slices (fp32 partial sums + ordered reduction), and on the four-wave 64x64
+    tile it runs on small grids of whole tiles."""
     M, N, K = shape
     plan = hgemm_lib.auto_plan(M, N, K)
     assert tile in plan["kernel"] and (plan["splits"] > 1) == split, plan

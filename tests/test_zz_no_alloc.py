@@ -32,7 +32,7 @@ def _call(lib, symbol, A, B, M, N, K, gpu):
 
 
 # each pair: a shape whose plan keeps partial sums or padded operands in the workspace, then a smaller one
-PAIRS = [((1024, 1024, 4096), (256, 256, 8192)),          # K slices on 128x128 tiles, then on 64x64 tiles
+PAIRS = [((1024, 1024, 8192), (256, 256, 8192)),          # K slices on 128x128 tiles, then on 64x64 tiles
          ((7168, 7168, 2048), (64, 4096, 4096)),          # (no workspace: last round on smaller tiles), split-K small-M kernel
          ((7168, 7168, 7168), (512, 512, 8192)),          # last round of a large grid in K slices
          ((1111, 1111, 1111), (515, 1032, 1100)),         # zero-padded operand copies
@@ -74,7 +74,7 @@ def test_static_workspace_matches_heap_workspace(oracle, hgemm_lib, gpu, first, 
 
 def test_static_workspace_allocates_nothing_and_rejects_what_does_not_fit(oracle, hgemm_lib, gpu):
     import torch
-    M, N, K = 1024, 1024, 4096
+    M, N, K = 1024, 1024, 8192
     assert hgemm_lib.auto_workspace_bytes(M, N, K)["partial"] > 0
     A, B = _to_gpu(oracle.fill((M, K), 93, 1), gpu), _to_gpu(oracle.fill((N, K), 93, 2), gpu)
     _call(hgemm_lib, "hgemm_auto_static_workspace", A, B, M, N, K, gpu)        # code object and scratch are resident now
