@@ -195,7 +195,7 @@ constexpr Candidate CANDIDATES[] = {
     {KERNEL_R256x128, 256, 128, 1, 3, 4.25, 0.476, 0.856},
     {KERNEL_MID128, 128, 128, 1, 5, 3.17, 0.266, 0.510},
     {KERNEL_SMALL64, 64, 64, 3, 3, 1.39, 0.294, 0.585},
-    // whole tiles only, no K slices; fitted on 16 to 256 tiles (256^3 ... 1024^3, K to 4096), where it is 13-22 % ahead of
+    // whole tiles only; fitted on 16 to 256 tiles (256^3 ... 1024^3, K to 4096), where it is 13-22 % ahead of
     // the one-wave tile; modelled at one workgroup per CU, which keeps it out of larger grids (where it is behind)
     {KERNEL_SMALL64_W4, 64, 64, 1, 3, 1.94, 0.216, 0.246},
 };
@@ -310,10 +310,9 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
         const bool whole_tiles_only = c.kernel == KERNEL_SMALL64_W4;
         if (whole_tiles_only && (M % c.bm || N % c.bn)) continue;
         for (int s = 1; s <= 32; s *= 2) {
-            if (whole_tiles_only && s > 1) break;
-            // whole 64x64 tiles, at most one per CU, no K slices: the four-wave tile is ahead of the one-wave tile on
+            // whole 64x64 tiles, at most one workgroup per CU: the four-wave tile is ahead of the one-wave tile on
             // every such grid that was measured (the model, fitted on larger grids, flatters the one-wave tile there)
-            if (c.kernel == KERNEL_SMALL64 && s == 1 && M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) <= cus) continue;
+            if (c.kernel == KERNEL_SMALL64 && M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) * (size_t)s <= cus) continue;
             if (K % ((size_t)s * 64) || K / s < (size_t)64 * c.stages) break;
             if (s > 1 && (size_t)s * slice_bytes > limits.partial_bytes) break;
             const double t = predict_us(c, M, N, K, s, cus);
@@ -465,7 +464,16 @@ void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, 
         case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128_S4: launch_pipelined<Mid128S4>(A, B, C, M, N, K, "hgemm_auto"); break;
         case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p, ws); break;
-        case KERNEL_SMALL64_W4: launch_tiled<Small64W4>(A, B, C, M, N, K, "hgemm_auto"); break;
+        case KERNEL_SMALL64_W4:
+            if (p.splits <= 1) {
+                launch_tiled<Small64W4>(A, B, C, M, N, K, "hgemm_auto");
+            } else {
+                check_operands(A, B, C, M, N, K);
+                HGEMM_CHECK(ws.partial != nullptr && ws.partial_bytes >= (size_t)p.splits * M * N * sizeof(float));
+                launch_tiled_split<Small64W4>(A, B, ws.partial, M, N, K, p.splits, "hgemm_auto");
+                launch_splitk_reduce(ws.partial, reinterpret_cast<half_t *>(C), M * N, p.splits);
+            }
+            break;
         case KERNEL_SPLIT_32x64: launch_splitk<Split32x64>(A, B, C, M, N, K, p.splits, ws); break;
         case KERNEL_SPLIT_64x64: launch_splitk<Split64x64>(A, B, C, M, N, K, p.splits, ws); break;
         case KERNEL_SPLIT_64x128: launch_splitk<Split64x128>(A, B, C, M, N, K, p.splits, ws); break;

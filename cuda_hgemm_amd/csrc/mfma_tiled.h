@@ -161,10 +161,12 @@ __device__ __forceinline__ void store_tile_via_lds(const floatx16 (&acc)[Cfg::TM
     }
 }
 
-template <class Cfg>
+// SPLIT: workgroup (x, y) computes K slice y (k_len wide) of tile x and leaves fp32 partial sums in
+// partial[y][M][N] for the ordered reduction; otherwise k_len == K and C is written.
+template <class Cfg, bool SPLIT = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
-    hgemm_tiled_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C, int M,
-                       int N, int K, int tiles_m, int tiles_n) {
+    hgemm_tiled_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
+                       float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, KSTEPS = Cfg::KSTEPS, CPR = Cfg::CPR;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES, THREADS = Cfg::THREADS;
@@ -180,9 +182,10 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     int tile_m, tile_n;
     tile_of_workgroup(blocked_order(N, K), 0, (int)blockIdx.x, (int)gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
 
-    const half_t *Ag = A + (size_t)tile_m * BM * K;
-    const half_t *Bg = B + (size_t)tile_n * BN * K;
-    const int num_k = K / BK;
+    const int k_begin = SPLIT ? (int)blockIdx.y * k_len : 0;
+    const half_t *Ag = A + (size_t)tile_m * BM * K + k_begin;
+    const half_t *Bg = B + (size_t)tile_n * BN * K + k_begin;
+    const int num_k = k_len / BK;
 
     // ---------------- global -> LDS copy set-up ----------------
     // REG: thread t moves chunk (row = t / CPR + it * THREADS/CPR, ch = t % CPR).
@@ -352,6 +355,24 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         }
     }
 
+    if constexpr (SPLIT) {
+        // Lane l holds row l % 32 of each 32x32 tile and, per register group g, four consecutive n at
+        // 8 g + 4 (l / 32): 16 bytes of an fp32 partial sum.
+        float *dst = partial + ((size_t)blockIdx.y * M + tile_m * BM + wm * Cfg::WM + (lane & 31)) * N + tile_n * BN +
+                     wn * Cfg::WN + ((lane >> 5) << 2);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    floatx4 v;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] = acc[i][j][g * 4 + r];
+                    *reinterpret_cast<floatx4 *>(dst + (size_t)(i * 32) * N + j * 32 + g * 8) = v;
+                }
+        return;
+    }
     // ---------------- epilogue: accumulators -> fp16 -> C ----------------
     __syncthreads();
     store_tile_via_lds<Cfg>(acc, lds, C, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN, wave, lane);
@@ -374,8 +395,30 @@ void launch_tiled(const void *A, const void *B, void *C, size_t M, size_t N, siz
     (void)configured;
     const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
     hgemm_tiled_kernel<Cfg><<<dim3(tiles_m * tiles_n), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
-        reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
-        (int)M, (int)N, (int)K, tiles_m, tiles_n);
+        reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), nullptr,
+        (int)M, (int)N, (int)K, (int)K, tiles_m, tiles_n);
+    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+}
+
+// K in `splits` slices: fp32 partial sums of slice s go to partial[s][M][N]; the caller runs the ordered reduction.
+template <class Cfg>
+void launch_tiled_split(const void *A, const void *B, float *partial, size_t M, size_t N, size_t K, int splits,
+                        const char *name) {
+    HGEMM_CHECK(splits >= 1 && K % (size_t)splits == 0 && partial != nullptr && splits <= 65535);
+    const size_t k_len = K / (size_t)splits;
+    HGEMM_CHECK_MSG(Cfg::supports(M, N, k_len),
+                    "%s (K in %d slices) needs M %% %d == 0, N %% %d == 0, slice %% %d == 0, slice >= %d (got M=%zu N=%zu K=%zu)",
+                    name, splits, Cfg::BM, Cfg::BN, Cfg::BK, Cfg::BK * (Cfg::STAGES > 1 ? Cfg::STAGES - 1 : 1), M, N, K);
+    static bool configured = [] {
+        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_tiled_kernel<Cfg, true>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        return true;
+    }();
+    (void)configured;
+    const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
+    hgemm_tiled_kernel<Cfg, true><<<dim3(tiles_m * tiles_n, splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
+        reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), nullptr, partial, (int)M, (int)N, (int)K,
+        (int)k_len, tiles_m, tiles_n);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 

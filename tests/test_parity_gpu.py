@@ -247,6 +247,7 @@ def test_auto_16384_sampled_rows(oracle, hgemm_lib, gpu):
     ((3072, 3072, 256), "192x192x64", False), ((2560, 2560, 256), "256x128x64", False),
     ((256, 256, 8192), "64x64x64", True), ((1024, 1024, 8192), "128x128x64", True),
     ((1024, 1024, 4096), "tiled 64x64x64", False), ((512, 768, 640), "tiled 64x64x64", False), ((192, 192, 192), "tiled 64x64x64", False),
+    ((512, 512, 4096), "tiled 64x64x64", True), ((256, 256, 16384), "tiled 64x64x64", True),
     ((512, 512, 8192), "64x64x64", True), ((1536, 1536, 16384), "192x192x64", True),
     ((2048, 2048, 16384), "256x256x64", True)])
 def test_auto_every_tile_with_and_without_k_slices(oracle, hgemm_lib, gpu, shape, tile, split):
