@@ -35,7 +35,7 @@ HGEMM_FN = C.CFUNCTYPE(None, *_HGEMM_ARGS)
 KERNEL_SYMBOLS = [
     "hgemm_simt_naive", "hgemm_mfma_naive", "hgemm_mfma_base", "hgemm_mfma_padding", "hgemm_mfma_swizzle",
     "hgemm_mfma_async", "hgemm_mfma_async_pg2s", "hgemm_mfma_async_pg2s_ps2r", "hgemm_mfma_async_stage2",
-    "hgemm_mfma_async_stage3", "hgemm_mfma_async_stage4", "hgemm_mfma_pipelined_64x64",
+    "hgemm_mfma_async_stage3", "hgemm_mfma_async_stage4", "hgemm_mfma_tiled_64x64", "hgemm_mfma_pipelined_64x64",
     "hgemm_mfma_pipelined_128x128", "hgemm_mfma_pipelined_192x192", "hgemm_mfma_pipelined_256x128",
     "hgemm_mfma_pipelined_256x256", "hgemm_mfma_chained_192x192", "hgemm_mfma_chained_256x128",
     "hgemm_mfma_chained_256x256", "hgemm_skinny", "hgemm_auto",

@@ -12,6 +12,7 @@ HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_pg2s_ps2r);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_stage2);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_stage3);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_async_stage4);
+HGEMM_DECLARE_SUPPORTS(hgemm_mfma_tiled_64x64);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_64x64);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_128x128);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_pipelined_192x192);
@@ -51,6 +52,8 @@ const Variant kVariants[] = {
     {"Mfma-Async-Stage2", "hgemm_mfma_async_stage2", hgemm_mfma_async_stage2, hgemm_mfma_async_stage2_supports, 1},
     {"Mfma-Async-Stage3", "hgemm_mfma_async_stage3", hgemm_mfma_async_stage3, hgemm_mfma_async_stage3_supports, 1},
     {"Mfma-Async-Stage4", "hgemm_mfma_async_stage4", hgemm_mfma_async_stage4, hgemm_mfma_async_stage4_supports, 1},
+    // the ladder's kernel on the small tile hgemm_auto uses for small grids
+    {"Mfma-Tiled-64x64", "hgemm_mfma_tiled_64x64", hgemm_mfma_tiled_64x64, hgemm_mfma_tiled_64x64_supports, 1},
     // the tuned kernel, one entry per tile, smallest first: the ladder ends at its fastest rung,
     // as the reference's run ends at mmaAsyncStage4 (src/main.cu:123)
     {"Mfma-Pipelined-64x64", "hgemm_mfma_pipelined_64x64", hgemm_mfma_pipelined_64x64,

@@ -139,7 +139,7 @@ using Tile192 = PipeConfig<192, 192, 64, 2, 2, 3, 16>;
 using Rect256x128 = PipeConfig<256, 128, 64, 2, 2, 3, 16>;
 // 64x64x64 on four waves (one 32x32 MFMA tile each) with the ladder's kernel: a small tile whose chunk takes a quarter
 // of the one-wave tile's matrix-pipe time; for grids that give a CU at most one tile
-using Small64W4 = TileConfig<64, 64, 64, 2, 2, 3, LOAD_DMA, LDS_SWIZZLE, true>;
+using Small64W4 = TileConfig<64, 64, 64, 2, 2, 3, LOAD_DMA, LDS_SWIZZLE, true>;  // also the entry point hgemm_mfma_tiled_64x64
 
 // Pipelined kernel with K cut into `splits` slices: fp32 partial sums per slice, then the
 // ordered reduction (the same one the small-M kernel uses), so the result is bit-identical

@@ -80,6 +80,11 @@ HGEMM_FUNC(hgemm_mfma_async_pg2s_ps2r);
 HGEMM_FUNC(hgemm_mfma_async_stage2);
 HGEMM_FUNC(hgemm_mfma_async_stage3);
 HGEMM_FUNC(hgemm_mfma_async_stage4);
+/* The ladder's kernel on a small tile: 64x64x64, four waves of one 32x32 MFMA tile each, 3-stage
+ * direct-to-LDS ring.  hgemm_auto runs it on grids of at most one whole tile per CU (the small
+ * squares of the sweep), where a launch is all latency.  Needs M % 64 == 0, N % 64 == 0,
+ * K % 64 == 0, K >= 128.  No counterpart in the reference, whose tiles are all 256x128. */
+HGEMM_FUNC(hgemm_mfma_tiled_64x64);
 
 /* The tuned CDNA4 kernel, one entry point per tile: K chunks of 64 in a ring of LDS buffers
  * filled by direct-to-LDS copies, v_mfma_f32_16x16x32_f16 with a hand-laid issue order,

@@ -48,9 +48,9 @@ def test_registry(hgemm_lib):
     names = [v["name"] for v in variants]
     assert names[0] == "Simt-Naive" and "Mfma-Async-Stage4" in names and names[-1] == "Auto"
     # the tuned kernel is selectable by name and closes the ladder (reference src/main.cu:123)
-    assert names.index("Mfma-Pipelined-256x256") == names.index("Mfma-Async-Stage4") + 5
+    assert names.index("Mfma-Pipelined-256x256") == names.index("Mfma-Async-Stage4") + 6
     assert names.index("Mfma-Chained-256x256") == names.index("Mfma-Pipelined-256x256") + 3 == len(names) - 3
-    assert all(v["default_run"] for v in variants if v["name"].startswith(("Mfma-Pipelined-", "Mfma-Chained-")))
+    assert all(v["default_run"] for v in variants if v["name"].startswith(("Mfma-Pipelined-", "Mfma-Chained-", "Mfma-Tiled-")))
     assert len(set(names)) == len(names)
     for v in variants:
         assert hgemm_lib.find(v["name"]) == v["index"] == hgemm_lib.find(v["symbol"])

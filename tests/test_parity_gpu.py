@@ -50,7 +50,8 @@ def _assert_close(oracle, got, ref_bits, K, ref_f32=None):
 
 
 TILED = ["hgemm_mfma_base", "hgemm_mfma_padding", "hgemm_mfma_swizzle", "hgemm_mfma_async", "hgemm_mfma_async_pg2s",
-         "hgemm_mfma_async_pg2s_ps2r", "hgemm_mfma_async_stage2", "hgemm_mfma_async_stage3", "hgemm_mfma_async_stage4"]
+         "hgemm_mfma_async_pg2s_ps2r", "hgemm_mfma_async_stage2", "hgemm_mfma_async_stage3", "hgemm_mfma_async_stage4",
+         "hgemm_mfma_tiled_64x64"]
 PIPELINED = ["hgemm_mfma_pipelined_64x64", "hgemm_mfma_pipelined_128x128", "hgemm_mfma_pipelined_192x192",
              "hgemm_mfma_pipelined_256x128", "hgemm_mfma_pipelined_256x256", "hgemm_mfma_chained_192x192",
              "hgemm_mfma_chained_256x128", "hgemm_mfma_chained_256x256"]
@@ -171,9 +172,10 @@ def test_ladder_rings_at_minimum_k(oracle, hgemm_lib, gpu, variant):
     on), and one K chunk more."""
     M, N = 512, 256
     kmin = min(k for k in (32, 64, 96, 128, 160) if hgemm_lib.supports(variant, M, N, k))
-    expected = {"hgemm_mfma_async_stage2": 64, "hgemm_mfma_async_stage3": 64, "hgemm_mfma_async_stage4": 96}.get(variant, 32)
+    expected = {"hgemm_mfma_async_stage2": 64, "hgemm_mfma_async_stage3": 64, "hgemm_mfma_async_stage4": 96,
+                "hgemm_mfma_tiled_64x64": 128}.get(variant, 32)
     assert kmin == expected, (variant, kmin)
-    step = 64 if variant == "hgemm_mfma_async_stage2" else 32      # its K chunk is 64 wide
+    step = 64 if variant in ("hgemm_mfma_async_stage2", "hgemm_mfma_tiled_64x64") else 32      # their K chunk is 64 wide
     for K in (kmin, kmin + step):
         At, Bt = oracle.fill((M, K), 61, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 61, 2, oracle.TERNARY, 0, 1)
         assert np.array_equal(_run(hgemm_lib, variant, At, Bt, gpu), oracle.hgemm(At, Bt)), K
