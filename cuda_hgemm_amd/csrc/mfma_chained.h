@@ -534,27 +534,16 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     }
     wait_vmcnt<0>();  // the redundant copies of the last iterations: landed before LDS is reused or the wave ends
     if constexpr (SPLIT) {
-        // a lane holds four consecutive n of row m = lane % 16 of each 16x16 tile: 16 bytes of fp32
-        const int row = tile_m * BM + wm * Cfg::WM + lane_late % MI, col = tile_n * BN + wn * Cfg::WN + (lane_late / MI) * 4;
-        if (tail_tiles > 0) {  // compact: whole tiles, nothing to guard
-            float *dst = partial + ((size_t)blockIdx.y * tail_tiles + slot) * (BM * BN) +
-                         (wm * Cfg::WM + lane_late % MI) * BN + wn * Cfg::WN + (lane_late / MI) * 4;
-            static_for<TM>([&](auto i_c) {
-                static_for<TN>([&](auto j_c) {
-                    constexpr int i = decltype(i_c)::value, j = decltype(j_c)::value;
-                    *reinterpret_cast<floatx4 *>(dst + (i * MI) * BN + j * MI) = AccTile<j * TM + i>::read();
-                });
-            });
-        } else {
-            float *dst = partial + ((size_t)blockIdx.y * M + row) * N + col;
-            static_for<TM>([&](auto i_c) {
-                static_for<TN>([&](auto j_c) {
-                    constexpr int i = decltype(i_c)::value, j = decltype(j_c)::value;
-                    if (!EDGE || (row + i * MI < M && col + j * MI < N))
-                        *reinterpret_cast<floatx4 *>(dst + (size_t)(i * MI) * N + j * MI) = AccTile<j * TM + i>::read();
-                });
-            });
-        }
+        __syncthreads();  // every wave has read its last operands: the strips reuse the ring
+        auto get = [&](auto i_c, auto j_c) -> floatx4 { return AccTile<decltype(j_c)::value * TM + decltype(i_c)::value>::read(); };
+        const int row0 = tile_m * BM + wm * Cfg::WM, col0 = tile_n * BN + wn * Cfg::WN;
+        if (tail_tiles > 0)  // compact: whole tiles [slice][slot][BM][BN], nothing to guard
+            store_wave_tile_f32<Cfg, false>(get, lds, partial + ((size_t)blockIdx.y * tail_tiles + slot) * (BM * BN) +
+                                                          (size_t)(wm * Cfg::WM) * BN + wn * Cfg::WN,
+                                            BN, BM, BN, wave, lane_late);
+        else
+            store_wave_tile_f32<Cfg, EDGE>(get, lds, partial + ((size_t)blockIdx.y * M + row0) * N + col0, N, M - row0,
+                                           N - col0, wave, lane_late);
     } else {
         (void)partial;
         __syncthreads();

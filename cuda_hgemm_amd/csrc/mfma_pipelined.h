@@ -226,6 +226,45 @@ __device__ __forceinline__ void store_wave_tile(const Acc (&acc)[Cfg::PTM][Cfg::
     }
 }
 
+// fp32 partial sums of a wave tile (16x16x32 accumulators: a lane holds four consecutive n of row m = lane % 16 of
+// each tile) -> memory, through LDS like the fp16 tile above: stored straight from that layout an instruction writes
+// sixteen 16-byte pieces of sixteen different rows; parked in the wave's strip 16 rows at a time and read back
+// row-contiguous, it writes whole 128-byte lines.  `get(i, j)` returns accumulator tile (i, j); `dst` is element (0, 0)
+// of the wave tile in a matrix with `ld` floats per row; rows >= rows_valid and 4-column pieces at or beyond
+// cols_valid (both relative to the wave tile) are not stored when EDGE.
+template <class Cfg, bool EDGE, class Get>
+__device__ __forceinline__ void store_wave_tile_f32(Get get, unsigned char *lds, float *__restrict__ dst, size_t ld,
+                                                    int rows_valid, int cols_valid, int wave, int lane) {
+    constexpr int MI = 16, TM = Cfg::PTM, TN = Cfg::PTN, WN = Cfg::WN;
+    static_assert(Cfg::MI == 16, "written for the 16x16x32 accumulator layout");
+    constexpr int STRIP_ROW_BYTES = WN * 4 + 16;
+    static_assert(MI * STRIP_ROW_BYTES <= Cfg::C_STRIP_BYTES, "the fp16 strip of a wave holds 16 rows of fp32");
+    constexpr int LANES_PER_ROW = WN / 4;                               // 16-byte pieces per row
+    constexpr int ROWS_PER_READ = 64 / LANES_PER_ROW;                   // lanes beyond that many rows idle
+    constexpr int READS = (MI + ROWS_PER_READ - 1) / ROWS_PER_READ;
+    constexpr bool EXACT = (64 % LANES_PER_ROW == 0) && (MI % ROWS_PER_READ == 0);
+    unsigned char *strip = lds + wave * Cfg::C_STRIP_BYTES;
+    unsigned char *wr = strip + (lane % MI) * STRIP_ROW_BYTES + ((lane / MI) << 4);
+    const int rd_row = lane / LANES_PER_ROW, rd_col = lane % LANES_PER_ROW;
+    const unsigned char *rd = strip + rd_row * STRIP_ROW_BYTES + rd_col * 16;
+    float *out = dst + (size_t)rd_row * ld + rd_col * 4;
+    static_for<TM>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        static_for<TN>([&](auto j_c) {
+            constexpr int j = decltype(j_c)::value;
+            *reinterpret_cast<floatx4 *>(wr + j * MI * 4) = get(i_c, j_c);
+        });
+#pragma unroll
+        for (int it = 0; it < READS; ++it) {
+            if (EXACT || (rd_row < ROWS_PER_READ && it * ROWS_PER_READ + rd_row < MI)) {
+                const floatx4 v = *reinterpret_cast<const floatx4 *>(rd + it * ROWS_PER_READ * STRIP_ROW_BYTES);
+                if (!EDGE || (i * MI + it * ROWS_PER_READ + rd_row < rows_valid && rd_col * 4 < cols_valid))
+                    *reinterpret_cast<floatx4 *>(out + (size_t)(i * MI + it * ROWS_PER_READ) * ld) = v;
+            }
+        }
+    });
+}
+
 // EDGE: M and N need not be multiples of the tile (N % 8 == 0 still, for aligned rows of
 // C).  Copies of rows beyond the matrix are redirected to its last row -- valid memory,
 // products never stored -- which costs nothing inside the loop; only the stores are guarded.
@@ -577,27 +616,16 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         c_epi = clock64();
     }
     if constexpr (SPLIT) {
-        // a lane holds four consecutive n of row m = lane % 16 of each 16x16 tile: 16 bytes of fp32
-        const int row = tile_m * BM + wm * Cfg::WM + lane % MI, col = tile_n * BN + wn * Cfg::WN + (lane / MI) * 4;
-        if (tail_tiles > 0) {  // compact: whole tiles, nothing to guard
-            float *dst = partial + ((size_t)blockIdx.y * tail_tiles + slot) * (BM * BN) +
-                         (wm * Cfg::WM + lane % MI) * BN + wn * Cfg::WN + (lane / MI) * 4;
-            static_for<TM>([&](auto i_c) {
-                static_for<TN>([&](auto j_c) {
-                    constexpr int i = decltype(i_c)::value, j = decltype(j_c)::value;
-                    *reinterpret_cast<floatx4 *>(dst + (i * MI) * BN + j * MI) = acc[i][j];
-                });
-            });
-        } else {
-            float *dst = partial + ((size_t)blockIdx.y * M + row) * N + col;
-            static_for<TM>([&](auto i_c) {
-                static_for<TN>([&](auto j_c) {
-                    constexpr int i = decltype(i_c)::value, j = decltype(j_c)::value;
-                    if (!EDGE || (row + i * MI < M && col + j * MI < N))
-                        *reinterpret_cast<floatx4 *>(dst + (size_t)(i * MI) * N + j * MI) = acc[i][j];
-                });
-            });
-        }
+        __syncthreads();  // every wave has read its last operands: the strips reuse the ring
+        auto get = [&](auto i_c, auto j_c) -> floatx4 { return acc[decltype(i_c)::value][decltype(j_c)::value]; };
+        const int row0 = tile_m * BM + wm * Cfg::WM, col0 = tile_n * BN + wn * Cfg::WN;
+        if (tail_tiles > 0)  // compact: whole tiles [slice][slot][BM][BN], nothing to guard
+            store_wave_tile_f32<Cfg, false>(get, lds, partial + ((size_t)blockIdx.y * tail_tiles + slot) * (BM * BN) +
+                                                          (size_t)(wm * Cfg::WM) * BN + wn * Cfg::WN,
+                                            BN, BM, BN, wave, lane);
+        else
+            store_wave_tile_f32<Cfg, EDGE>(get, lds, partial + ((size_t)blockIdx.y * M + row0) * N + col0, N, M - row0,
+                                           N - col0, wave, lane);
     } else {
         (void)partial;
         __syncthreads();
