@@ -138,8 +138,15 @@ using Small64 = PipeConfig<64, 64, 64, 1, 1, 3, 16>;
 using Tile192 = PipeConfig<192, 192, 64, 2, 2, 3, 16>;
 using Rect256x128 = PipeConfig<256, 128, 64, 2, 2, 3, 16>;
 // 64x64x64 on four waves (one 32x32 MFMA tile each) with the ladder's kernel: a small tile whose chunk takes a quarter
-// of the one-wave tile's matrix-pipe time; for grids that give a CU at most one tile
-using Small64W4 = TileConfig<64, 64, 64, 2, 2, 3, LOAD_DMA, LDS_SWIZZLE, true>;  // also the entry point hgemm_mfma_tiled_64x64
+// of the one-wave tile's matrix-pipe time; for grids that give a CU at most one tile.  Three forms by the number of
+// chunks a workgroup walks: the plain 3-stage ring up to 4 (the look-ahead prologue costs more than it returns),
+// the look-ahead loop on 5 stages (also the entry point hgemm_mfma_tiled_64x64; 4 stages are 1-2 % ahead while the
+// operands sit in L2 and 15-25 % behind once they do not: 512 x 512 x 4096), and on 6 stages from 40 chunks
+// (K >= 2560 per slice), where one more chunk in flight pays.
+using Small64W4Short = TileConfig<64, 64, 64, 2, 2, 3, LOAD_DMA, LDS_SWIZZLE, true>;
+using Small64W4 = TileConfig<64, 64, 64, 2, 2, 5, LOAD_DMA, LDS_SWIZZLE, true, true>;
+using Small64W4Deep = TileConfig<64, 64, 64, 2, 2, 6, LOAD_DMA, LDS_SWIZZLE, true, true>;
+constexpr size_t W4_SHORT_MAX_CHUNKS = 4, W4_DEEP_MIN_CHUNKS = 40;
 
 // Pipelined kernel with K cut into `splits` slices: fp32 partial sums per slice, then the
 // ordered reduction (the same one the small-M kernel uses), so the result is bit-identical
@@ -195,12 +202,21 @@ constexpr Candidate CANDIDATES[] = {
     {KERNEL_R256x128, 256, 128, 1, 3, 4.25, 0.476, 0.856},
     {KERNEL_MID128, 128, 128, 1, 5, 3.17, 0.266, 0.510},
     {KERNEL_SMALL64, 64, 64, 3, 3, 1.39, 0.294, 0.585},
-    // whole tiles only; fitted on 16 to 256 tiles (256^3 ... 1024^3, K to 4096), where it is 13-22 % ahead of
-    // the one-wave tile; modelled at one workgroup per CU, which keeps it out of larger grids (where it is behind)
-    {KERNEL_SMALL64_W4, 64, 64, 1, 3, 1.94, 0.216, 0.246},
+    // whole tiles only, at most one workgroup per CU (larger grids are kept from it below: it is behind there);
+    // fitted on 16 to 256 workgroups, K = 256 to 16384, in the forms run_plan picks by the length of a slice
+    {KERNEL_SMALL64_W4, 64, 64, 1, 3, 2.40, 0.168, 0.195},
 };
-// launch; reduction kernel: fixed + per slice + fp32 partials written and read back
-constexpr double LAUNCH_US = 0.16, REDUCE_US = 3.90, REDUCE_SLICE_US = 0.10, REDUCE_BYTES_PER_US = 7040e3;
+// launch; reduction kernel: fixed + per slice + fp32 partials written and read back.  Partial sums of a few MB
+// come back from the L2s: measured 3.0 us behind the same kernel at 2.4 MB against 4.5-5 us at 4.2 MB, and twice
+// the slices cost nothing there.  (Refitted with K-sliced launches dealt slice-major: 2.8-7.4 us for 2-17 MB.)
+constexpr double LAUNCH_US = 0.16, REDUCE_US = 3.00, REDUCE_SLICE_US = 0.10, REDUCE_BYTES_PER_US = 8700e3;
+constexpr double REDUCE_SMALL_US = 2.40, REDUCE_SMALL_SLICE_US = 0.05, REDUCE_SMALL_BYTES = 3e6;
+double reduce_us(int slices, double elems) {
+    const double bytes = (double)slices * elems * 4.0;
+    const bool small = bytes <= REDUCE_SMALL_BYTES;
+    return (small ? REDUCE_SMALL_US : REDUCE_US) + (small ? REDUCE_SMALL_SLICE_US : REDUCE_SLICE_US) * slices +
+           2.0 * bytes / REDUCE_BYTES_PER_US;
+}
 // extra cost of finishing a grid with a separate launch for its last round: in K slices / on smaller tiles
 constexpr double TAIL_US = 3.6, TAIL_SUB_US = 4.4;
 size_t padded_n(size_t N) { return (N + 7) / 8 * 8; }
@@ -218,8 +234,7 @@ double predict_us(const Candidate &c, size_t M, size_t N, size_t K, int splits, 
     const size_t full = wgs / slots, rem = wgs % slots;
     double t = LAUNCH_US + (double)full * (c.fix + chunks * c.hi);
     if (rem) t += c.fix + chunks * (c.lo + (c.hi - c.lo) * (double)rem / (double)slots);
-    if (splits > 1)
-        t += REDUCE_US + REDUCE_SLICE_US * splits + (double)splits * (double)M * (double)N * 8.0 / REDUCE_BYTES_PER_US;
+    if (splits > 1) t += reduce_us(splits, (double)M * (double)N);
     return t;
 }
 
@@ -232,7 +247,7 @@ double predict_tail_us(const Candidate &c, size_t M, size_t N, size_t K, int ts,
     const double chunks = (double)(K / 64);
     double t = LAUNCH_US + (double)full * (c.fix + chunks * c.hi);
     t += LAUNCH_US + c.fix + chunks / ts * (c.lo + (c.hi - c.lo) * (double)(rem * ts) / (double)slots);
-    t += REDUCE_US + REDUCE_SLICE_US * ts + (double)ts * (double)rem * c.bm * c.bn * 8.0 / REDUCE_BYTES_PER_US + TAIL_US;
+    t += reduce_us(ts, (double)rem * c.bm * c.bn) + TAIL_US;
     return t;
 }
 
@@ -310,6 +325,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
         const bool whole_tiles_only = c.kernel == KERNEL_SMALL64_W4;
         if (whole_tiles_only && (M % c.bm || N % c.bn)) continue;
         for (int s = 1; s <= 32; s *= 2) {
+            if (whole_tiles_only && (M / c.bm) * (N / c.bn) * (size_t)s > cus) break;
             // whole 64x64 tiles, at most one workgroup per CU: the four-wave tile is ahead of the one-wave tile on
             // every such grid that was measured (the model, fitted on larger grids, flatters the one-wave tile there)
             if (c.kernel == KERNEL_SMALL64 && M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) * (size_t)s <= cus) continue;
@@ -464,16 +480,28 @@ void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, 
         case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128_S4: launch_pipelined<Mid128S4>(A, B, C, M, N, K, "hgemm_auto"); break;
         case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p, ws); break;
-        case KERNEL_SMALL64_W4:
+        case KERNEL_SMALL64_W4: {
+            const size_t chunks = K / 64 / (size_t)(p.splits > 1 ? p.splits : 1);
             if (p.splits <= 1) {
-                launch_tiled<Small64W4>(A, B, C, M, N, K, "hgemm_auto");
+                if (chunks <= W4_SHORT_MAX_CHUNKS)
+                    launch_tiled<Small64W4Short>(A, B, C, M, N, K, "hgemm_auto");
+                else if (chunks < W4_DEEP_MIN_CHUNKS)
+                    launch_tiled<Small64W4>(A, B, C, M, N, K, "hgemm_auto");
+                else
+                    launch_tiled<Small64W4Deep>(A, B, C, M, N, K, "hgemm_auto");
             } else {
                 check_operands(A, B, C, M, N, K);
                 HGEMM_CHECK(ws.partial != nullptr && ws.partial_bytes >= (size_t)p.splits * M * N * sizeof(float));
-                launch_tiled_split<Small64W4>(A, B, ws.partial, M, N, K, p.splits, "hgemm_auto");
+                if (chunks <= W4_SHORT_MAX_CHUNKS)
+                    launch_tiled_split<Small64W4Short>(A, B, ws.partial, M, N, K, p.splits, "hgemm_auto");
+                else if (chunks < W4_DEEP_MIN_CHUNKS)
+                    launch_tiled_split<Small64W4>(A, B, ws.partial, M, N, K, p.splits, "hgemm_auto");
+                else
+                    launch_tiled_split<Small64W4Deep>(A, B, ws.partial, M, N, K, p.splits, "hgemm_auto");
                 launch_splitk_reduce(ws.partial, reinterpret_cast<half_t *>(C), M * N, p.splits);
             }
             break;
+        }
         case KERNEL_SPLIT_32x64: launch_splitk<Split32x64>(A, B, C, M, N, K, p.splits, ws); break;
         case KERNEL_SPLIT_64x64: launch_splitk<Split64x64>(A, B, C, M, N, K, p.splits, ws); break;
         case KERNEL_SPLIT_64x128: launch_splitk<Split64x128>(A, B, C, M, N, K, p.splits, ws); break;
@@ -653,7 +681,7 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
         case KERNEL_MID128: return "pipelined 128x128x64, 4 waves, 5-stage ring";
         case KERNEL_MID128_S4: return "pipelined 128x128x64, 4 waves, 4-stage ring";
         case KERNEL_SMALL64: return "pipelined 64x64x64, 1 wave, 3-stage ring";
-        case KERNEL_SMALL64_W4: return "tiled 64x64x64, 4 waves of 32x32, 3-stage ring";
+        case KERNEL_SMALL64_W4: return "tiled 64x64x64, 4 waves of 32x32, look-ahead ring";
         case KERNEL_T192: return "pipelined 192x192x64, 4 waves, 3-stage ring";
         case KERNEL_R256x128: return "pipelined 256x128x64, 4 waves, 3-stage ring";
         case KERNEL_SPLIT_32x64: return "split-K 32x64x64, 2 waves, 4-stage ring";

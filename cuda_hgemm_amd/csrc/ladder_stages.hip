@@ -8,6 +8,7 @@ using namespace hgemm;
 HGEMM_DEFINE_TILED_VARIANT(hgemm_mfma_async_stage2, 256, 128, 64, 4, 2, 2, LOAD_DMA, LDS_SWIZZLE, true)
 HGEMM_DEFINE_TILED_VARIANT(hgemm_mfma_async_stage3, 256, 128, 32, 4, 2, 3, LOAD_DMA, LDS_SWIZZLE, true)
 HGEMM_DEFINE_TILED_VARIANT(hgemm_mfma_async_stage4, 256, 128, 32, 4, 2, 4, LOAD_DMA, LDS_SWIZZLE, true)
-// The same kernel on a 64x64x64 tile, four waves of one 32x32 MFMA tile each, 3-stage ring: what
-// hgemm_auto runs on small grids of whole tiles (no counterpart in the reference, whose tiles are 256x128).
-HGEMM_DEFINE_TILED_VARIANT(hgemm_mfma_tiled_64x64, 64, 64, 64, 2, 2, 3, LOAD_DMA, LDS_SWIZZLE, true)
+// The same kernel on a 64x64x64 tile, four waves of one 32x32 MFMA tile each, 5-stage ring with the barrier one
+// chunk ahead and whole chunks of operands in registers: what hgemm_auto runs on small grids of whole tiles
+// (no counterpart in the reference, whose tiles are 256x128).
+HGEMM_DEFINE_TILED_VARIANT(hgemm_mfma_tiled_64x64, 64, 64, 64, 2, 2, 5, LOAD_DMA, LDS_SWIZZLE, true, true)

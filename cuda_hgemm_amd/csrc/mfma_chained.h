@@ -142,9 +142,17 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     int tile_m, tile_n;
     // the same in every launch that works on this problem (probe builds can force either order)
     const bool blocked = (Cfg::DBG & 16) ? false : ((Cfg::DBG & 32) ? true : blocked_order(N, K));
-    // this workgroup's slot among the launch's gridDim.x: slots are dealt so that the workgroups an XCD runs
-    // together are neighbours in the tile order
-    const int slot = slot_of_workgroup(blocked, (int)blockIdx.x, (int)gridDim.x);
+    // this workgroup's slot among the launch's positions: slots are dealt so that the workgroups an XCD runs
+    // together are neighbours in the tile order.  A K-sliced launch is one-dimensional as well, slice-major, so
+    // that those neighbours also work on the same slice of K.
+    int slot, slice = 0;
+    if constexpr (SPLIT) {
+        const int slices = K / k_len;
+        slice_and_slot_of_workgroup((int)blockIdx.x, (int)gridDim.x / slices, slices, slice, slot);
+        slice = __builtin_amdgcn_readfirstlane(slice);
+    } else {
+        slot = slot_of_workgroup(blocked, (int)blockIdx.x, (int)gridDim.x);
+    }
     if (subdiv == 0) {
         // the launch covers positions [first_block, first_block + gridDim.x) of the tile order
         tile_of_position(blocked, first_block + slot, tiles_m, tiles_n, tile_m, tile_n);
@@ -162,7 +170,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     tile_m = __builtin_amdgcn_readfirstlane(tile_m);  // wave-uniform by construction: keep them in SGPRs
     tile_n = __builtin_amdgcn_readfirstlane(tile_n);
     const int num_k = k_len / BK;
-    const int k_begin = SPLIT ? (int)blockIdx.y * k_len : 0;
+    const int k_begin = slice * k_len;
 
     // ---- copy set-up: wave w, instruction i fills LDS rows [(i*WAVES + w)*ROWS_PER_DMA, +ROWS_PER_DMA)
     const unsigned char *a_base = reinterpret_cast<const unsigned char *>(A + (size_t)tile_m * BM * K + k_begin);
@@ -538,11 +546,11 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         auto get = [&](auto i_c, auto j_c) -> floatx4 { return AccTile<decltype(j_c)::value * TM + decltype(i_c)::value>::read(); };
         const int row0 = tile_m * BM + wm * Cfg::WM, col0 = tile_n * BN + wn * Cfg::WN;
         if (tail_tiles > 0)  // compact: whole tiles [slice][slot][BM][BN], nothing to guard
-            store_wave_tile_f32<Cfg, false>(get, lds, partial + ((size_t)blockIdx.y * tail_tiles + slot) * (BM * BN) +
+            store_wave_tile_f32<Cfg, false>(get, lds, partial + ((size_t)slice * tail_tiles + slot) * (BM * BN) +
                                                           (size_t)(wm * Cfg::WM) * BN + wn * Cfg::WN,
                                             BN, BM, BN, wave, lane_late);
         else
-            store_wave_tile_f32<Cfg, EDGE>(get, lds, partial + ((size_t)blockIdx.y * M + row0) * N + col0, N, M - row0,
+            store_wave_tile_f32<Cfg, EDGE>(get, lds, partial + ((size_t)slice * M + row0) * N + col0, N, M - row0,
                                            N - col0, wave, lane_late);
     } else {
         (void)partial;

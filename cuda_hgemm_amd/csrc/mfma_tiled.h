@@ -17,10 +17,14 @@
 //           SWIZZLE (XOR of the 16-byte chunk index with the row, reference mma_permuted.cu:105-108)
 //   STAGES  LDS ring depth (reference mma_async_stage4.cu:52 K_STAGE)
 //   FRAG_PREFETCH  double-buffered operand registers (reference mma_async_pg2s_ps2r.cu:184-185)
+//   LOOKAHEAD  (no counterpart in the reference) the barrier of an iteration confirms the *next* chunk, so the
+//           operand double buffer runs across chunk boundaries and no LDS read latency is exposed behind a barrier
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "common.h"
 #include "tile_order.h"
@@ -39,12 +43,12 @@ enum { LOAD_REG = 0, LOAD_DMA = 1 };
 enum { LDS_LINEAR = 0, LDS_PADDED = 1, LDS_SWIZZLE = 2 };
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int LOADER_, int LAYOUT_,
-          bool FRAG_PREFETCH_>
+          bool FRAG_PREFETCH_, bool LOOKAHEAD_ = false>
 struct TileConfig {
     static constexpr int BM = BM_, BN = BN_, BK = BK_;
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int STAGES = STAGES_, LOADER = LOADER_, LAYOUT = LAYOUT_;
-    static constexpr bool FRAG_PREFETCH = FRAG_PREFETCH_;
+    static constexpr bool FRAG_PREFETCH = FRAG_PREFETCH_, LOOKAHEAD = LOOKAHEAD_;
 
     static constexpr int WAVES = WAVES_M * WAVES_N;
     static constexpr int THREADS = WAVES * 64;
@@ -72,9 +76,11 @@ struct TileConfig {
     static_assert(LOADER == LOAD_REG || LAYOUT != LDS_PADDED, "direct-to-LDS rows are contiguous: no padding");
     static_assert(LOADER == LOAD_REG || (A_BYTES % (1024 * WAVES) == 0 && B_BYTES % (1024 * WAVES) == 0),
                   "direct-to-LDS copy must divide evenly over the waves");
-    static_assert(STAGES >= 1 && STAGES <= 5, "1..5 LDS stages");
+    static_assert(STAGES >= 1 && STAGES <= 10, "1..10 LDS stages");
     static_assert(LDS_BYTES <= 160 * 1024, "exceeds the 160 KB LDS of a gfx950 CU");
     static_assert((STAGES - 1) * LOADS_PER_STAGE <= 63, "vmcnt is a 6-bit counter");
+    static_assert(!LOOKAHEAD || (LOADER == LOAD_DMA && FRAG_PREFETCH && STAGES >= 3 && KSTEPS % 2 == 0),
+                  "the look-ahead loop is written for the direct-to-LDS ring with double-buffered operands");
 
     static bool supports(size_t M, size_t N, size_t K) {
         return M % BM == 0 && N % BN == 0 && K % BK == 0 && K >= (size_t)BK * (STAGES > 1 ? STAGES - 1 : 1);
@@ -161,8 +167,9 @@ __device__ __forceinline__ void store_tile_via_lds(const floatx16 (&acc)[Cfg::TM
     }
 }
 
-// SPLIT: workgroup (x, y) computes K slice y (k_len wide) of tile x and leaves fp32 partial sums in
-// partial[y][M][N] for the ordered reduction; otherwise k_len == K and C is written.
+// SPLIT: a one-dimensional launch of tiles x slices workgroups; each computes one K slice (k_len wide) of one tile
+// and leaves fp32 partial sums in partial[slice][M][N] for the ordered reduction; otherwise k_len == K and C is
+// written.
 template <class Cfg, bool SPLIT = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_tiled_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
@@ -179,10 +186,17 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
 
-    int tile_m, tile_n;
-    tile_of_workgroup(blocked_order(N, K), 0, (int)blockIdx.x, (int)gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+    int tile_m, tile_n, slice = 0;
+    if constexpr (SPLIT) {
+        int slot;
+        slice_and_slot_of_workgroup((int)blockIdx.x, tiles_m * tiles_n, K / k_len, slice, slot);
+        tile_of_position(blocked_order(N, K), slot, tiles_m, tiles_n, tile_m, tile_n);
+        slice = __builtin_amdgcn_readfirstlane(slice);
+    } else {
+        tile_of_workgroup(blocked_order(N, K), 0, (int)blockIdx.x, (int)gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+    }
 
-    const int k_begin = SPLIT ? (int)blockIdx.y * k_len : 0;
+    const int k_begin = slice * k_len;
     const half_t *Ag = A + (size_t)tile_m * BM * K + k_begin;
     const half_t *Bg = B + (size_t)tile_n * BN * K + k_begin;
     const int num_k = k_len / BK;
@@ -331,6 +345,62 @@ __global__ void __launch_bounds__(Cfg::THREADS)
                 compute_stage(0);
                 __syncthreads();
             }
+        } else if constexpr (Cfg::LOOKAHEAD) {
+            // Ring of STAGES buffers, barrier one chunk ahead, whole chunks of operands in registers.  At the top
+            // of iteration kt every operand of chunk kt is already on its way into registers; the wait and the
+            // barrier confirm chunk kt+1 (and retire every wave's reads of chunk kt-1, whose buffer the new copy
+            // refills), then the wave issues all operand reads of chunk kt+1, the copy of chunk kt+STAGES-1, and
+            // only then the MFMAs of chunk kt.  With one or two MFMAs per k-step (small wave tiles) a read issued one
+            // step ahead is still in flight when its MFMA comes up; a chunk ahead, LDS latency is off the chain.
+#pragma unroll
+            for (int s = 0; s < STAGES - 1; ++s) dma_fetch(s, s);  // supports() guarantees num_k >= STAGES-1
+            wait_vmcnt<(STAGES - 2) * L>();
+            __syncthreads();
+            half8 af[2][KSTEPS][TM], bf[2][KSTEPS][TN];
+            auto load_chunk = [&](int stage, half8 (&a)[KSTEPS][TM], half8 (&b)[KSTEPS][TN]) {
+#pragma unroll
+                for (int kk = 0; kk < KSTEPS; ++kk) load_frags(stage, kk, a[kk], b[kk]);
+            };
+            load_chunk(0, af[0], bf[0]);
+            int cur = 0, fill = STAGES - 1;
+            // STEADY: the copy of chunk kt+STAGES-1 exists (so does chunk kt+1, and the wait count is the full one);
+            // the last iterations (the odd one left by the unrolled pairs and those after the last copy) take their
+            // decisions at run time.
+            auto iteration = [&](auto steady, int kt, half8 (&ca)[KSTEPS][TM], half8 (&cb)[KSTEPS][TN],
+                                 half8 (&na)[KSTEPS][TM], half8 (&nb)[KSTEPS][TN]) {
+                constexpr bool STEADY = decltype(steady)::value;
+                const int nxt = (cur + 1 == STAGES) ? 0 : cur + 1;
+                if (STEADY || kt + 1 < num_k) {
+                    // copies issued so far: chunks up to min(kt+STAGES-2, num_k-1); all but those beyond kt+1 must land
+                    if (STEADY || num_k - 1 - (kt + 1) >= STAGES - 3) {
+                        wait_vmcnt<(STAGES - 3) * L>();
+                    } else {
+                        wait_vmcnt<0>();
+                    }
+                    // a bare barrier: the fence of __syncthreads() would wait for this wave's own operand reads of
+                    // chunk kt, which nothing behind the barrier overwrites (the refilled buffer held chunk kt-1,
+                    // consumed by MFMAs already issued)
+                    __builtin_amdgcn_sched_barrier(0);  // the MFMAs of chunk kt-1 (and their waits) stay in front
+                    asm volatile("s_barrier" ::: "memory");
+                    load_chunk(nxt, na, nb);
+                }
+                if (STEADY || kt + STAGES - 1 < num_k) dma_fetch(kt + STAGES - 1, fill);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int kk = 0; kk < KSTEPS; ++kk) mma_step(ca[kk], cb[kk]);
+                cur = nxt;
+                fill = (fill + 1 == STAGES) ? 0 : fill + 1;
+            };
+            const int steady_end = num_k - (STAGES - 1);
+            int kt = 0;
+            for (; kt + 2 <= steady_end; kt += 2) {
+                iteration(std::true_type{}, kt, af[0], bf[0], af[1], bf[1]);
+                iteration(std::true_type{}, kt + 1, af[1], bf[1], af[0], bf[0]);
+            }
+            for (; kt < num_k; kt += 2) {
+                iteration(std::false_type{}, kt, af[0], bf[0], af[1], bf[1]);
+                if (kt + 1 < num_k) iteration(std::false_type{}, kt + 1, af[1], bf[1], af[0], bf[0]);
+            }
         } else {
             // Ring of STAGES buffers.  At the top of iteration kt the copies of chunks
             // kt .. kt+STAGES-2 are in flight; wait for the oldest, meet at the barrier
@@ -358,7 +428,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     if constexpr (SPLIT) {
         // Lane l holds row l % 32 of each 32x32 tile and, per register group g, four consecutive n at
         // 8 g + 4 (l / 32): 16 bytes of an fp32 partial sum.
-        float *dst = partial + ((size_t)blockIdx.y * M + tile_m * BM + wm * Cfg::WM + (lane & 31)) * N + tile_n * BN +
+        float *dst = partial + ((size_t)slice * M + tile_m * BM + wm * Cfg::WM + (lane & 31)) * N + tile_n * BN +
                      wn * Cfg::WN + ((lane >> 5) << 2);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -416,7 +486,8 @@ void launch_tiled_split(const void *A, const void *B, float *partial, size_t M, 
     }();
     (void)configured;
     const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
-    hgemm_tiled_kernel<Cfg, true><<<dim3(tiles_m * tiles_n, splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
+    HGEMM_CHECK((size_t)tiles_m * tiles_n * (size_t)splits < ((size_t)1 << 31));
+    hgemm_tiled_kernel<Cfg, true><<<dim3(tiles_m * tiles_n * splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), nullptr, partial, (int)M, (int)N, (int)K,
         (int)k_len, tiles_m, tiles_n);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());

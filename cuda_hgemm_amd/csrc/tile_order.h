@@ -109,4 +109,14 @@ HGEMM_HOST_DEVICE void tile_of_workgroup(bool blocked, int first, int b, int cou
     tile_of_position(blocked, first + slot_of_workgroup(blocked, b, count), tiles_m, tiles_n, tile_m, tile_n);
 }
 
+// K-sliced launches are one-dimensional too: `count` positions times `slices`, slice-major, dealt in contiguous
+// shares like a strip launch.  An XCD then works on whole slices, or on a run of neighbouring tiles of one slice,
+// and the panels it streams are shared by the workgroups it runs together; with the slice as the launch's second
+// dimension an XCD would get every slice of a few tiles, whose K ranges share nothing.
+HGEMM_HOST_DEVICE void slice_and_slot_of_workgroup(int b, int count, int slices, int &slice, int &slot) {
+    const int p = xcd_contiguous(b, count * slices);
+    slice = p / count;
+    slot = p - slice * count;
+}
+
 }  // namespace hgemm

@@ -80,10 +80,12 @@ HGEMM_FUNC(hgemm_mfma_async_pg2s_ps2r);
 HGEMM_FUNC(hgemm_mfma_async_stage2);
 HGEMM_FUNC(hgemm_mfma_async_stage3);
 HGEMM_FUNC(hgemm_mfma_async_stage4);
-/* The ladder's kernel on a small tile: 64x64x64, four waves of one 32x32 MFMA tile each, 3-stage
- * direct-to-LDS ring.  hgemm_auto runs it on grids of at most one whole tile per CU (the small
- * squares of the sweep), where a launch is all latency.  Needs M % 64 == 0, N % 64 == 0,
- * K % 64 == 0, K >= 128.  No counterpart in the reference, whose tiles are all 256x128. */
+/* The ladder's kernel on a small tile: 64x64x64, four waves of one 32x32 MFMA tile each, 5-stage
+ * direct-to-LDS ring whose barrier confirms the chunk after the one being multiplied, so a whole
+ * chunk of operands is in registers before its MFMAs start.  hgemm_auto runs it on grids of at
+ * most one whole tile per CU (the small squares of the sweep), where a launch is all latency.
+ * Needs M % 64 == 0, N % 64 == 0, K % 64 == 0, K >= 256.  No counterpart in the reference, whose
+ * tiles are all 256x128. */
 HGEMM_FUNC(hgemm_mfma_tiled_64x64);
 
 /* The tuned CDNA4 kernel, one entry point per tile: K chunks of 64 in a ring of LDS buffers

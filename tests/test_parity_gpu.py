@@ -171,9 +171,9 @@ def test_ladder_rings_at_minimum_k(oracle, hgemm_lib, gpu, variant):
     starts draining at once: the branch that waits for every copy from the first iteration
     on), and one K chunk more."""
     M, N = 512, 256
-    kmin = min(k for k in (32, 64, 96, 128, 160) if hgemm_lib.supports(variant, M, N, k))
+    kmin = min(k for k in (32, 64, 96, 128, 160, 192, 256) if hgemm_lib.supports(variant, M, N, k))
     expected = {"hgemm_mfma_async_stage2": 64, "hgemm_mfma_async_stage3": 64, "hgemm_mfma_async_stage4": 96,
-                "hgemm_mfma_tiled_64x64": 128}.get(variant, 32)
+                "hgemm_mfma_tiled_64x64": 256}.get(variant, 32)
     assert kmin == expected, (variant, kmin)
     step = 64 if variant in ("hgemm_mfma_async_stage2", "hgemm_mfma_tiled_64x64") else 32      # their K chunk is 64 wide
     for K in (kmin, kmin + step):
@@ -181,6 +181,17 @@ def test_ladder_rings_at_minimum_k(oracle, hgemm_lib, gpu, variant):
         assert np.array_equal(_run(hgemm_lib, variant, At, Bt, gpu), oracle.hgemm(At, Bt)), K
         A, B = oracle.fill((M, K), 62, 1), oracle.fill((N, K), 62, 2)
         _assert_close(oracle, _run(hgemm_lib, variant, A, B, gpu), oracle.hgemm(A, B), K)
+
+
+@pytest.mark.parametrize("chunks", [5, 6, 7, 8, 9, 12, 13])
+def test_lookahead_ring_every_chunk_count(oracle, hgemm_lib, gpu, chunks):
+    """hgemm_mfma_tiled_64x64 walks K in unrolled pairs of iterations while a copy is still to be issued, then one
+    iteration at a time: odd and even counts of either kind, exact on ternary inputs."""
+    M, N, K = 192, 320, 64 * chunks
+    At, Bt = oracle.fill((M, K), 63, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 63, 2, oracle.TERNARY, 0, 1)
+    assert np.array_equal(_run(hgemm_lib, "hgemm_mfma_tiled_64x64", At, Bt, gpu), oracle.hgemm(At, Bt))
+    A, B = oracle.fill((M, K), 64, 1), oracle.fill((N, K), 64, 2)
+    _assert_close(oracle, _run(hgemm_lib, "hgemm_mfma_tiled_64x64", A, B, gpu), oracle.hgemm(A, B), K)
 
 
 def test_vendor_comparator_matches_the_checker(oracle, vendor_lib, gpu):
@@ -247,7 +258,7 @@ def test_auto_16384_sampled_rows(oracle, hgemm_lib, gpu):
 
 @pytest.mark.parametrize("shape,tile,split", [
     ((3072, 3072, 256), "192x192x64", False), ((2560, 2560, 256), "256x128x64", False),
-    ((256, 256, 8192), "64x64x64", True), ((1024, 1024, 8192), "128x128x64", True),
+    ((256, 256, 8192), "64x64x64", True), ((1024, 1024, 16384), "128x128x64", True),
     ((1024, 1024, 4096), "tiled 64x64x64", False), ((512, 768, 640), "tiled 64x64x64", False), ((192, 192, 192), "tiled 64x64x64", False),
     ((512, 512, 4096), "tiled 64x64x64", True), ((256, 256, 16384), "tiled 64x64x64", True),
     ((512, 512, 8192), "64x64x64", True), ((1536, 1536, 16384), "192x192x64", True),

@@ -44,6 +44,27 @@ PROGRAM = textwrap.dedent(
                             return printf("tile: order %%d grid %%d x %%d position %%d\n", blocked, tm, tn, p), 1;
                     }
                 }
+        // K-sliced launches: every (slice, slot) pair exactly once, and the 32 workgroups an XCD runs together in a
+        // launch of 64 tiles x 4 slices stay inside one slice
+        for (int count = 1; count <= 300; ++count)
+            for (int slices = 1; slices <= 32; slices += (slices < 4 ? 1 : 7)) {
+                std::vector<int> seen(count * slices, 0);
+                for (int b = 0; b < count * slices; ++b) {
+                    int slice = -1, slot = -1;
+                    slice_and_slot_of_workgroup(b, count, slices, slice, slot);
+                    if (slice < 0 || slice >= slices || slot < 0 || slot >= count || seen[slice * count + slot]++)
+                        return printf("slices: count %%d slices %%d workgroup %%d\n", count, slices, b), 1;
+                }
+            }
+        for (int x = 0; x < 8; ++x) {
+            std::set<int> slices_of_xcd;
+            for (int w = 0; w < 32; ++w) {
+                int slice, slot;
+                slice_and_slot_of_workgroup(w * 8 + x, 64, 4, slice, slot);
+                slices_of_xcd.insert(slice);
+            }
+            if (slices_of_xcd.size() != 1) return printf("slices: XCD %%d works on %%zu slices\n", x, slices_of_xcd.size()), 1;
+        }
         // a launch that covers positions [first, first + count): the tiles of head and tail launches are disjoint
         for (int blocked = 0; blocked < 2; ++blocked) {
             const int tm = 17, tn = 23, total = tm * tn, head = 256;
