@@ -101,6 +101,7 @@ __device__ __forceinline__ void store_chained_tile(unsigned char *lds, half_t *_
             for (int r = 0; r < 4; ++r) v[r] = (half_t)acc[r];
             *reinterpret_cast<half4 *>(wr + (j * MI) * 2) = v;
         });
+        wave_lds_exchange_point();
 #pragma unroll
         for (int it = 0; it < READS; ++it) {
             if (EXACT || (rd_row < ROWS_PER_READ && it * ROWS_PER_READ + rd_row < MI)) {
@@ -109,6 +110,7 @@ __device__ __forceinline__ void store_chained_tile(unsigned char *lds, half_t *_
                     *reinterpret_cast<u32x4 *>(cp + (size_t)(i * MI + it * ROWS_PER_READ) * N) = v;
             }
         }
+        wave_lds_exchange_point();
     });
 }
 

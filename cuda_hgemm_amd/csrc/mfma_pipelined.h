@@ -215,6 +215,7 @@ __device__ __forceinline__ void store_wave_tile(const Acc (&acc)[Cfg::PTM][Cfg::
                 for (int r = 0; r < 4; ++r) v[r] = (half_t)acc[i][j][g * 4 + r];
                 *reinterpret_cast<half4 *>(wr + (j * MI + g * 8) * 2) = v;
             }
+        wave_lds_exchange_point();
 #pragma unroll
         for (int it = 0; it < READS; ++it) {
             if (EXACT || (rd_row < ROWS_PER_READ && it * ROWS_PER_READ + rd_row < MI)) {
@@ -223,6 +224,7 @@ __device__ __forceinline__ void store_wave_tile(const Acc (&acc)[Cfg::PTM][Cfg::
                     *reinterpret_cast<u32x4 *>(cp + (size_t)(i * MI + it * ROWS_PER_READ) * N) = v;
             }
         }
+        wave_lds_exchange_point();
     }
 }
 
@@ -254,6 +256,7 @@ __device__ __forceinline__ void store_wave_tile_f32(Get get, unsigned char *lds,
             constexpr int j = decltype(j_c)::value;
             *reinterpret_cast<floatx4 *>(wr + j * MI * 4) = get(i_c, j_c);
         });
+        wave_lds_exchange_point();
 #pragma unroll
         for (int it = 0; it < READS; ++it) {
             if (EXACT || (rd_row < ROWS_PER_READ && it * ROWS_PER_READ + rd_row < MI)) {
@@ -262,6 +265,7 @@ __device__ __forceinline__ void store_wave_tile_f32(Get get, unsigned char *lds,
                     *reinterpret_cast<floatx4 *>(out + (size_t)(i * MI + it * ROWS_PER_READ) * ld) = v;
             }
         }
+        wave_lds_exchange_point();
     });
 }
 

@@ -124,6 +124,13 @@ __device__ __forceinline__ int swizzle_of_row(int row) {
     return ((line & 7) ^ ((line >> 3) & 1)) & (Cfg::CPR - 1);
 }
 
+// Lanes of one wave exchange data through LDS in the epilogues below.  The hardware executes a wave's LDS
+// instructions in order, so no wait is needed between a store and the load that picks the data up in another lane;
+// but the compiler reasons lane by lane: where it can prove that the bytes a lane stores and the bytes the same lane
+// loads never coincide, it is free to issue the load first (it did, for some tile shapes: stale strip contents in
+// the output).  An empty ordered statement that claims to touch memory keeps stores and loads on their own sides.
+__device__ __forceinline__ void wave_lds_exchange_point() { asm volatile("" ::: "memory"); }
+
 // Epilogue shared by the tiled kernels: accumulators -> fp16 -> C, staged through LDS.
 // A lane of the (operand-swapped) accumulator holds four consecutive n of one row; stored
 // straight to global memory that is 16 useful bytes per 32 rows per instruction, i.e. a
@@ -159,11 +166,13 @@ __device__ __forceinline__ void store_tile_via_lds(const floatx16 (&acc)[Cfg::TM
                 for (int r = 0; r < 4; ++r) v[r] = (half_t)acc[i][j][g * 4 + r];
                 *reinterpret_cast<half4 *>(wr + (j * 32 + g * 8) * 2) = v;
             }
+        wave_lds_exchange_point();
 #pragma unroll
         for (int it = 0; it < READS; ++it) {
             const u32x4 v = *reinterpret_cast<const u32x4 *>(rd + it * ROWS_PER_READ * STRIP_ROW_BYTES);
             *reinterpret_cast<u32x4 *>(cp + (size_t)(i * 32 + it * ROWS_PER_READ) * N) = v;
         }
+        wave_lds_exchange_point();
     }
 }
 

@@ -262,7 +262,8 @@ def test_auto_16384_sampled_rows(oracle, hgemm_lib, gpu):
     ((1024, 1024, 4096), "tiled 64x64x64", False), ((512, 768, 640), "tiled 64x64x64", False), ((192, 192, 192), "tiled 64x64x64", False),
     ((512, 512, 4096), "tiled 64x64x64", True), ((256, 256, 16384), "tiled 64x64x64", True),
     ((512, 512, 8192), "64x64x64", True), ((1536, 1536, 16384), "192x192x64", True),
-    ((2048, 2048, 16384), "256x256x64", True)])
+    ((2048, 2048, 16384), "256x256x64", True), ((1536, 1536, 8192), "192x192x64", True),
+    ((2048, 2048, 10240), "256x128x64", True)])
 def test_auto_every_tile_with_and_without_k_slices(oracle, hgemm_lib, gpu, shape, tile, split):
     """Shapes chosen so the dispatcher's cost model lands on each pipelined tile, alone and
     with K cut into slices (fp32 partial sums + ordered reduction), and on the four-wave 64x64
@@ -278,6 +279,17 @@ def test_auto_every_tile_with_and_without_k_slices(oracle, hgemm_lib, gpu, shape
     ref = oracle.hgemm(At, Bt)
     assert np.abs(ref.view(np.float16).astype(np.float32)).max() <= 2048      # integers exact in fp16
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), ref)
+
+
+@pytest.mark.parametrize("t", [768, 1280, 1536, 1792, 2048, 2304])
+@pytest.mark.parametrize("K", [7168, 10240, 13312, 16384])
+def test_auto_deep_k_plans(oracle, hgemm_lib, gpu, t, K):
+    """Squares of few tiles under a deep K: the dispatcher cuts K into slices on every tile, with either tuned
+    kernel (the shapes cover 128x128, 192x192, 256x128 and 256x256, interleaved and chained).  Slabs of 16 complete
+    rows are checked, so every row of an MFMA tile and every lane of the wave that stores it is looked at."""
+    A, B = oracle.fill((t, K), 71, 1), oracle.fill((t, K), 71, 2)
+    got = _run(hgemm_lib, "hgemm_auto", A, B, gpu)
+    _sampled_check(oracle, got, A, B, K, rows_per_slab=16, slabs=3, seed=t + K)
 
 
 @pytest.mark.parametrize("shape,mode", [((7168, 7168, 7168), "k slices"), ((7168, 7168, 2048), "128x128x64"),
