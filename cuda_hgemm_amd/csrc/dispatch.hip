@@ -134,6 +134,9 @@ using Split128x128 = SkinnyConfig<128, 128, 2, 2, 4>;
 using Big256 = PipeConfig<256, 256, 64, 2, 2, 2, 16, 0, 1>;
 using Mid128 = PipeConfig<128, 128, 64, 2, 2, 5, 16>;
 using Mid128S4 = PipeConfig<128, 128, 64, 2, 2, 4, 16>;
+// two LDS buffers (64 KB): two workgroups fit a CU, and one's C tile goes out while the other multiplies.  Pays where
+// a workgroup's K loop is shorter than its epilogue and C outgrows the Infinity Cache: 16384^2 x 256 201 -> 170 us.
+using Mid128S2 = PipeConfig<128, 128, 64, 2, 2, 2, 16>;
 using Small64 = PipeConfig<64, 64, 64, 1, 1, 3, 16>;
 using Tile192 = PipeConfig<192, 192, 64, 2, 2, 3, 16>;
 using Rect256x128 = PipeConfig<256, 128, 64, 2, 2, 3, 16>;
@@ -202,6 +205,8 @@ constexpr Candidate CANDIDATES[] = {
     {KERNEL_R256x128, 256, 128, 1, 3, 4.25, 0.476, 0.856},
     {KERNEL_MID128, 128, 128, 1, 5, 3.17, 0.266, 0.510},
     {KERNEL_SMALL64, 64, 64, 3, 3, 1.39, 0.294, 0.585},
+    // K of at most four chunks only (kept to that below); fitted on 8192^2 ... 16384^2 x 256
+    {KERNEL_MID128_S2, 128, 128, 2, 2, 1.77, 0.60, 0.885},
     // whole tiles only, at most one workgroup per CU (larger grids are kept from it below: it is behind there);
     // fitted on 16 to 256 workgroups, K = 256 to 16384, in the forms run_plan picks by the length of a slice
     {KERNEL_SMALL64_W4, 64, 64, 1, 3, 2.40, 0.168, 0.195},
@@ -326,6 +331,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
         if (whole_tiles_only && (M % c.bm || N % c.bn)) continue;
         for (int s = 1; s <= 32; s *= 2) {
             if (whole_tiles_only && (M / c.bm) * (N / c.bn) * (size_t)s > cus) break;
+            if (c.kernel == KERNEL_MID128_S2 && (s > 1 || K > 256)) break;
             // whole 64x64 tiles, at most one workgroup per CU: the four-wave tile is ahead of the one-wave tile on
             // every such grid that was measured (the model, fitted on larger grids, flatters the one-wave tile there)
             if (c.kernel == KERNEL_SMALL64 && M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) * (size_t)s <= cus) continue;
@@ -346,7 +352,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
         // a grid of whole rounds plus a few workgroups: run those few in K slices
         const size_t wgs = div_ceil(M, (size_t)c.bm) * div_ceil(N, (size_t)c.bn), slots = cus * (size_t)c.per_cu;
         const size_t rem = wgs % slots;
-        if (wgs > slots && rem > 0 && !whole_tiles_only) {
+        if (wgs > slots && rem > 0 && !whole_tiles_only && c.kernel != KERNEL_MID128_S2) {
             for (int ts = 2; ts <= 16; ts *= 2) {
                 if (K % ((size_t)ts * 64) || K / ts < (size_t)64 * c.stages || rem * ts > slots) break;
                 if ((size_t)ts * rem * c.bm * c.bn * sizeof(float) > limits.partial_bytes) break;
@@ -364,7 +370,9 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
             }
             if (c.kernel == KERNEL_BIG256) {  // ... or on smaller tiles that divide this one
                 for (const Candidate &small : CANDIDATES) {
-                    if (small.kernel == KERNEL_BIG256 || small.kernel == KERNEL_SMALL64_W4 || c.bm % small.bm || c.bn % small.bn) continue;
+                    if (small.kernel == KERNEL_BIG256 || small.kernel == KERNEL_SMALL64_W4 || small.kernel == KERNEL_MID128_S2 ||
+                        c.bm % small.bm || c.bn % small.bn)
+                        continue;
                     if (K < (size_t)64 * small.stages) continue;
                     const double t = predict_subtile_us(c, small, M, N, K, cus);
                     if (p.kernel != KERNEL_NONE && t < best) {
@@ -479,6 +487,7 @@ void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, 
         case KERNEL_R256x128: launch_pipelined_plan<Rect256x128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128_S4: launch_pipelined<Mid128S4>(A, B, C, M, N, K, "hgemm_auto"); break;
+        case KERNEL_MID128_S2: launch_pipelined<Mid128S2>(A, B, C, M, N, K, "hgemm_auto"); break;
         case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_SMALL64_W4: {
             const size_t chunks = K / 64 / (size_t)(p.splits > 1 ? p.splits : 1);
@@ -680,6 +689,7 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
         case KERNEL_BIG256: return "pipelined 256x256x64, 4 waves, LDS ring 3 (A) + 2 (B)";
         case KERNEL_MID128: return "pipelined 128x128x64, 4 waves, 5-stage ring";
         case KERNEL_MID128_S4: return "pipelined 128x128x64, 4 waves, 4-stage ring";
+        case KERNEL_MID128_S2: return "pipelined 128x128x64, 4 waves, 2-stage ring";
         case KERNEL_SMALL64: return "pipelined 64x64x64, 1 wave, 3-stage ring";
         case KERNEL_SMALL64_W4: return "tiled 64x64x64, 4 waves of 32x32, look-ahead ring";
         case KERNEL_T192: return "pipelined 192x192x64, 4 waves, 3-stage ring";
