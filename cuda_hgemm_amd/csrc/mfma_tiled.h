@@ -17,8 +17,9 @@
 //           SWIZZLE (XOR of the 16-byte chunk index with the row, reference mma_permuted.cu:105-108)
 //   STAGES  LDS ring depth (reference mma_async_stage4.cu:52 K_STAGE)
 //   FRAG_PREFETCH  double-buffered operand registers (reference mma_async_pg2s_ps2r.cu:184-185)
-//   LOOKAHEAD  (no counterpart in the reference) the barrier of an iteration confirms the *next* chunk, so the
-//           operand double buffer runs across chunk boundaries and no LDS read latency is exposed behind a barrier
+//   LOOKAHEAD  (no counterpart in the reference) the barrier of an iteration confirms the *next* chunk, whose
+//           operands are all read into a second set of registers while the MFMAs of the current chunk run: for wave
+//           tiles of one or two MFMAs per k-step, where a read issued one step ahead is still in flight when needed
 #pragma once
 
 #include <hip/hip_runtime.h>
