@@ -149,6 +149,8 @@ using Rect256x128 = PipeConfig<256, 128, 64, 2, 2, 3, 16>;
 using Small64W4Short = TileConfig<64, 64, 64, 2, 2, 3, LOAD_DMA, LDS_SWIZZLE, true>;
 using Small64W4 = TileConfig<64, 64, 64, 2, 2, 5, LOAD_DMA, LDS_SWIZZLE, true, true>;
 using Small64W4Deep = TileConfig<64, 64, 64, 2, 2, 6, LOAD_DMA, LDS_SWIZZLE, true, true>;
+// two workgroups per CU (grids of one to two tiles per CU): the 4-stage form, 64 KB each, 0-6 % ahead of 5 stages there
+using Small64W4Pair = TileConfig<64, 64, 64, 2, 2, 4, LOAD_DMA, LDS_SWIZZLE, true, true>;
 constexpr size_t W4_SHORT_MAX_CHUNKS = 4, W4_DEEP_MIN_CHUNKS = 40;
 
 // Pipelined kernel with K cut into `splits` slices: fp32 partial sums per slice, then the
@@ -210,6 +212,10 @@ constexpr Candidate CANDIDATES[] = {
     // whole tiles only, at most one workgroup per CU (larger grids are kept from it below: it is behind there);
     // fitted on 16 to 256 workgroups, K = 256 to 16384, in the forms run_plan picks by the length of a slice
     {KERNEL_SMALL64_W4, 64, 64, 1, 3, 2.40, 0.168, 0.195},
+    // the same tile with two workgroups sharing a CU (its 5-stage form takes 80 KB of LDS): grids of one to two
+    // tiles per CU, unsliced, fewer than 40 chunks (kept to that below); fitted on 1088^2 ... 1408^2, K = 512 ... 2048,
+    // where it is 7-19 % ahead of the 128x128 and one-wave 64x64 tiles; from 2 x CUs + 1 tiles on it is far behind
+    {KERNEL_SMALL64_W4, 64, 64, 2, 3, 2.40, 0.10, 0.40},
 };
 // launch; reduction kernel: fixed + per slice + fp32 partials written and read back.  Partial sums of a few MB
 // come back from the L2s: measured 3.0 us behind the same kernel at 2.4 MB against 4.5-5 us at 4.2 MB, and twice
@@ -330,7 +336,11 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
         const bool whole_tiles_only = c.kernel == KERNEL_SMALL64_W4;
         if (whole_tiles_only && (M % c.bm || N % c.bn)) continue;
         for (int s = 1; s <= 32; s *= 2) {
-            if (whole_tiles_only && (M / c.bm) * (N / c.bn) * (size_t)s > cus) break;
+            if (whole_tiles_only) {
+                const size_t wgs = (M / c.bm) * (N / c.bn) * (size_t)s;
+                if (wgs > cus * (size_t)c.per_cu) break;
+                if (c.per_cu == 2 && (wgs <= cus || s > 1 || K / 64 >= W4_DEEP_MIN_CHUNKS)) break;
+            }
             if (c.kernel == KERNEL_MID128_S2 && (s > 1 || K > 256)) break;
             // whole 64x64 tiles, at most one workgroup per CU: the four-wave tile is ahead of the one-wave tile on
             // every such grid that was measured (the model, fitted on larger grids, flatters the one-wave tile there)
@@ -494,6 +504,8 @@ void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, 
             if (p.splits <= 1) {
                 if (chunks <= W4_SHORT_MAX_CHUNKS)
                     launch_tiled<Small64W4Short>(A, B, C, M, N, K, "hgemm_auto");
+                else if ((M / 64) * (N / 64) > (size_t)compute_units())
+                    launch_tiled<Small64W4Pair>(A, B, C, M, N, K, "hgemm_auto");
                 else if (chunks < W4_DEEP_MIN_CHUNKS)
                     launch_tiled<Small64W4>(A, B, C, M, N, K, "hgemm_auto");
                 else

@@ -260,7 +260,7 @@ def test_auto_16384_sampled_rows(oracle, hgemm_lib, gpu):
     ((3072, 3072, 256), "192x192x64", False), ((2560, 2560, 320), "256x128x64", False),
     ((4096, 4096, 256), "2-stage ring", False), ((4100, 4104, 192), "2-stage ring", False), ((2048, 2048, 128), "2-stage ring", False),
     ((256, 256, 8192), "64x64x64", True), ((1024, 1024, 16384), "128x128x64", True),
-    ((1024, 1024, 4096), "tiled 64x64x64", False), ((512, 768, 640), "tiled 64x64x64", False), ((192, 192, 192), "tiled 64x64x64", False),
+    ((1024, 1024, 4096), "tiled 64x64x64", False), ((512, 768, 640), "tiled 64x64x64", False), ((1152, 1280, 1024), "tiled 64x64x64", False), ((1408, 1408, 2048), "tiled 64x64x64", False), ((192, 192, 192), "tiled 64x64x64", False),
     ((512, 512, 4096), "tiled 64x64x64", True), ((256, 256, 16384), "tiled 64x64x64", True),
     ((512, 512, 8192), "64x64x64", True), ((1536, 1536, 16384), "192x192x64", True),
     ((2048, 2048, 16384), "256x256x64", True), ((1536, 1536, 8192), "192x192x64", True),
