@@ -111,6 +111,35 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
     assert plan(4095, 4095, 4095)["kernel"].startswith("zero-padded")          # large and unaligned
 
 
+def test_auto_plan_invariants_over_many_shapes(hgemm_lib):
+    """What run_plan relies on, for every plan the model can come up with (no launch, no GPU): K slices are whole
+    numbers of 64-wide chunks and fit the workspace cap; the four-wave 64x64 tile only takes grids of whole tiles, at
+    most two per CU, and is unsliced and below 40 chunks when two share a CU; the 2-stage 128x128 tile only takes
+    K <= 256, unsliced, without a tail."""
+    import random
+    rng = random.Random(5)
+    shapes = [(t, t, k) for t in range(64, 3073, 64) for k in (64, 128, 192, 256, 320, 1024, 2560, 4096, 16384)]
+    for _ in range(1500):
+        shapes.append((rng.randrange(1, 9000), 8 * rng.randrange(1, 1100), 64 * rng.randrange(1, 260)))
+    cus = 256
+    for (m, n, k) in shapes:
+        p = hgemm_lib.auto_plan(m, n, k)
+        s = p["splits"]
+        assert s >= 1 and p["tail_splits"] >= 1, (m, n, k, p)
+        if p["kernel"].startswith(("pipelined", "tiled", "split-K")):
+            assert k % (64 * s) == 0 and k % (64 * p["tail_splits"]) == 0, (m, n, k, p)
+        need = hgemm_lib.auto_workspace_bytes(m, n, k)
+        assert need["partial"] <= 512 << 20 and need["operands"] <= 1024 << 20, (m, n, k, need)
+        if p["kernel"].startswith("tiled 64x64x64"):
+            assert m % 64 == 0 and n % 64 == 0 and p["tail_tiles"] == 0, (m, n, k, p)
+            tiles = (m // 64) * (n // 64)
+            assert tiles * s <= 2 * cus and k // s >= 192, (m, n, k, p)
+            if tiles * s > cus:
+                assert s == 1 and k // 64 < 40, (m, n, k, p)
+        if "2-stage ring" in p["kernel"]:
+            assert k <= 256 and s == 1 and p["tail_tiles"] == 0, (m, n, k, p)
+
+
 def test_workspace_needs_of_auto_plans(hgemm_lib):
     """What hgemm_auto's plan keeps in device memory beyond A, B and C (no launch, no GPU)."""
     need = hgemm_lib.auto_workspace_bytes
