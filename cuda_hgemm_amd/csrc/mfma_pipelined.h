@@ -221,7 +221,7 @@ __device__ __forceinline__ void store_wave_tile(const Acc (&acc)[Cfg::PTM][Cfg::
             if (EXACT || (rd_row < ROWS_PER_READ && it * ROWS_PER_READ + rd_row < MI)) {
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(rd + it * ROWS_PER_READ * STRIP_ROW_BYTES);
                 if (!EDGE || (row0 + rd_row + i * MI + it * ROWS_PER_READ < M && col0 + rd_col * 8 < N))
-                    *reinterpret_cast<u32x4 *>(cp + (size_t)(i * MI + it * ROWS_PER_READ) * N) = v;
+                    store_streaming(reinterpret_cast<u32x4 *>(cp + (size_t)(i * MI + it * ROWS_PER_READ) * N), v);
             }
         }
         wave_lds_exchange_point();
@@ -695,7 +695,7 @@ __global__ void __launch_bounds__(256)
             v[e] = (half_t)s0[e];
             v[4 + e] = (half_t)s1[e];
         }
-        *reinterpret_cast<half8 *>(C + (size_t)row * N + col) = v;
+        store_streaming(reinterpret_cast<half8 *>(C + (size_t)row * N + col), v);
     }
 }
 

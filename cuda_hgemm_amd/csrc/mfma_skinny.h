@@ -179,7 +179,7 @@ __global__ void __launch_bounds__(256)
     hvec_t out;
 #pragma unroll
     for (int r = 0; r < VEC; ++r) out[r] = (half_t)acc[r];
-    *reinterpret_cast<hvec_t *>(C + i) = out;
+    store_streaming(reinterpret_cast<hvec_t *>(C + i), out);
 }
 
 // elems must be a multiple of 8 (every tile dimension is).
