@@ -101,7 +101,9 @@ template <class Cfg>
 void launch_splitk(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, int splits,
                    const Workspace &ws) {
     static bool configured = [] {
-        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_skinny_kernel<Cfg>),
+        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_skinny_kernel<Cfg, false>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_skinny_kernel<Cfg, true>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
         return true;
     }();
@@ -116,7 +118,11 @@ void launch_splitk(const void *A, const void *B, void *C, size_t M, size_t N, si
         HGEMM_CHECK(ws.partial != nullptr && ws.partial_bytes >= (size_t)splits * M * N * sizeof(float));
         partial = ws.partial;
     }
-    hgemm_skinny_kernel<Cfg><<<grid, dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
+    // a B of 48 MB or more is streamed past the caches: +2-12 % from 64 MB up (N = 8192 ... 28672 at K = 4096),
+    // 0-7 % slower at 32 MB (N = K = 4096), where the next call finds parts of B in the Infinity Cache otherwise
+    const bool stream_b = div_ceil(M, Cfg::BM) == 1 && N * K >= ((size_t)24 << 20);
+    auto kernel = stream_b ? &hgemm_skinny_kernel<Cfg, true> : &hgemm_skinny_kernel<Cfg, false>;
+    kernel<<<grid, dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
         partial, (int)M, (int)N, (int)K, (int)(K / splits), (int)tiles_n);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
@@ -133,7 +139,6 @@ using Split128x128 = SkinnyConfig<128, 128, 2, 2, 4>;
 // 256x256x64 tile on v_mfma_f32_16x16x32_f16, two B buffers and three A buffers (all 160 KB of LDS)
 using Big256 = PipeConfig<256, 256, 64, 2, 2, 2, 16, 0, 1>;
 using Mid128 = PipeConfig<128, 128, 64, 2, 2, 5, 16>;
-using Mid128S4 = PipeConfig<128, 128, 64, 2, 2, 4, 16>;
 // two LDS buffers (64 KB): two workgroups fit a CU, and one's C tile goes out while the other multiplies.  Pays where
 // a workgroup's K loop is shorter than its epilogue and C outgrows the Infinity Cache: 16384^2 x 256 201 -> 170 us.
 using Mid128S2 = PipeConfig<128, 128, 64, 2, 2, 2, 16>;
@@ -305,7 +310,10 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     if (M == 0 || N == 0 || K == 0) return p;
     const size_t cus = (size_t)compute_units();
     const size_t slice_bytes = M * N * sizeof(float);  // fp32 partial sums of one K slice of the whole product
-    if (M <= 8 && decode_supports(M, N, K)) {  // a few rows: one streaming pass over B, no second launch
+    // a few rows: one streaming pass over B, no second launch; against a B of 96 MB or more the split-K kernel with
+    // B streamed past the caches is ahead from M = 6 (N = 14336: 8-16 %, N = 28672: 2-3 %; K = 4096)
+    const bool large_b = N * K >= ((size_t)48 << 20);
+    if (M <= 8 && decode_supports(M, N, K) && !(M >= 6 && large_b && skinny_supports(M, N, K))) {
         int bn = 16, waves = 1;
         decode_plan(M, N, K, cus, &bn, &waves);
         p.kernel = bn == 16 ? KERNEL_DECODE_BN16 : KERNEL_DECODE_BN32;
@@ -313,10 +321,6 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
         return p;
     }
     if (skinny_supports(M, N, K)) {
-        if (M == 128 && N >= 8192 && N % 128 == 0 && Mid128S4::supports(M, N, K)) {
-            p.kernel = KERNEL_MID128_S4;
-            return p;
-        }
         const bool wide = M > 32 && N >= 16384 && N % 128 == 0;  // enough columns: 128-wide tiles stream B better
         if (M <= 32)
             p.kernel = KERNEL_SPLIT_32x64;
@@ -496,7 +500,6 @@ void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, 
         case KERNEL_T192: launch_pipelined_plan<Tile192>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_R256x128: launch_pipelined_plan<Rect256x128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p, ws); break;
-        case KERNEL_MID128_S4: launch_pipelined<Mid128S4>(A, B, C, M, N, K, "hgemm_auto"); break;
         case KERNEL_MID128_S2: launch_pipelined<Mid128S2>(A, B, C, M, N, K, "hgemm_auto"); break;
         case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_SMALL64_W4: {
@@ -700,7 +703,6 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
     switch (kernel) {
         case KERNEL_BIG256: return "pipelined 256x256x64, 4 waves, LDS ring 3 (A) + 2 (B)";
         case KERNEL_MID128: return "pipelined 128x128x64, 4 waves, 5-stage ring";
-        case KERNEL_MID128_S4: return "pipelined 128x128x64, 4 waves, 4-stage ring";
         case KERNEL_MID128_S2: return "pipelined 128x128x64, 4 waves, 2-stage ring";
         case KERNEL_SMALL64: return "pipelined 64x64x64, 1 wave, 3-stage ring";
         case KERNEL_SMALL64_W4: return "tiled 64x64x64, 4 waves of 32x32, look-ahead ring";

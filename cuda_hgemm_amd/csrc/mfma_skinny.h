@@ -22,7 +22,10 @@ namespace hgemm {
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_>
 struct SkinnyConfig : TileConfig<BM_, BN_, 64, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true> {};
 
-template <class Cfg>
+// STREAM_B: B is copied with the non-temporal hint.  Every byte of B is read once; when B is larger than the
+// Infinity Cache keeps (N = 28672, K = 4096: 235 MB) the hint is worth 11-12 % (M = 16 ... 64: 64.5 -> 72.6 %, 63.6 ->
+// 70.5 %, 57.6 -> 64.7 % of 8 TB/s), when B fits (N = K = 4096) it costs up to 7 %, so the launcher decides by size.
+template <class Cfg, bool STREAM_B = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_skinny_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
                         float *__restrict__ partial, int M, int N, int K, int k_per_split, int tiles_n) {
@@ -68,7 +71,10 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         for (int it = 0; it < Cfg::A_DMA; ++it) dma_load16(a_src[it] + koff, base + it * Cfg::WAVES * 1024);
 #pragma unroll
         for (int it = 0; it < Cfg::B_DMA; ++it)
-            dma_load16(b_src[it] + koff, base + Cfg::A_BYTES + it * Cfg::WAVES * 1024);
+            if constexpr (STREAM_B)
+                dma_load16_streaming(b_src[it] + koff, base + Cfg::A_BYTES + it * Cfg::WAVES * 1024);
+            else
+                dma_load16(b_src[it] + koff, base + Cfg::A_BYTES + it * Cfg::WAVES * 1024);
     };
 
     // ---- fragments

@@ -113,6 +113,17 @@ __device__ __forceinline__ void dma_load16(const void *gptr, uint32_t lds_addr) 
         : "memory");
 }
 
+// The same copy with the non-temporal hint, for operands that are read once (B of the small-M kernels).
+__device__ __forceinline__ void dma_load16_streaming(const void *gptr, uint32_t lds_addr) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, off nt"
+        :
+        : "s"(lds_addr), "v"(gptr)
+        : "memory");
+}
+
 // XOR applied to the 16-byte chunk index of LDS row `row` (rows are BK*2 bytes).
 // One 128-byte bank line holds 128/(BK*2) rows; consecutive bank lines get consecutive
 // XOR values, and bit 3 of the line index is folded in so that 16 consecutive lines

@@ -9,7 +9,6 @@ enum KernelId {
     KERNEL_NONE = 0,
     KERNEL_BIG256,      // pipelined 256x256x64, 4 waves
     KERNEL_MID128,      // pipelined 128x128x64, 4 waves, 5-stage ring
-    KERNEL_MID128_S4,   // pipelined 128x128x64, 4 waves, 4-stage ring (M = 128 against a very wide B)
     KERNEL_SMALL64,     // pipelined 64x64x64, 1 wave, 3-stage ring
     KERNEL_SPLIT_32x64,   // split-K family: BM x BN tile, 4-stage ring, M guarded
     KERNEL_SPLIT_64x64,

@@ -101,10 +101,10 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
     for m in (1, 8, 16, 64, 128):
         for n in (4096, 28672):
             p = plan(m, n, 4096)
-            if m <= 8:
+            if m <= 8 and not (m >= 6 and n == 28672):     # from M = 6 a B of 96 MB or more goes to the split-K kernel
                 assert p["kernel"].startswith("streaming decode"), (m, n, p)
             else:
-                assert p["kernel"].startswith("split-K") or (m == 128 and p["kernel"].startswith("pipelined 128x128")), (m, n, p)
+                assert p["kernel"].startswith("split-K"), (m, n, p)
             assert 4096 % (p["splits"] * 64) == 0
     assert plan(100, 100, 100)["kernel"].startswith("guarded 128x128x32")      # no tile divides it
     assert plan(1000, 4000, 4096)["kernel"].startswith("pipelined")            # ragged M, N: guarded edges

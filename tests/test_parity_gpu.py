@@ -354,9 +354,9 @@ def test_decode_shapes(oracle, hgemm_lib, gpu, M, N):
         assert np.array_equal(first, second)
 
 
-@pytest.mark.parametrize("shape", [(1, 4096, 4096), (2, 32, 256), (3, 96, 512), (5, 4096, 1024), (7, 28672, 2048),
+@pytest.mark.parametrize("shape", [(1, 4096, 4096), (2, 32, 256), (3, 96, 512), (5, 4096, 1024), (5, 28672, 2048),
                                    (8, 2048, 8192), (4, 16384, 4096), (8, 32768, 1280), (6, 64, 16384), (3, 64, 768),
-                                   (8, 20480, 2816)])
+                                   (4, 20480, 2816), (7, 8192, 4096)])
 def test_streaming_decode_kernel(oracle, hgemm_lib, gpu, shape):
     """M <= 8: both column-tile widths, one to eight K slices per workgroup, slices that are
     and are not a whole number of load groups."""
@@ -368,6 +368,20 @@ def test_streaming_decode_kernel(oracle, hgemm_lib, gpu, shape):
     _assert_close(oracle, first, oracle.hgemm(A, B), K)
     assert np.array_equal(first, second)
     At, Bt = oracle.fill((M, K), 32, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 32, 2, oracle.TERNARY, 0, 1)
+    assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
+
+
+@pytest.mark.parametrize("shape", [(7, 28672, 2048), (8, 20480, 2816), (6, 14336, 4096), (100, 14336, 4096)])
+def test_small_m_against_a_large_b(oracle, hgemm_lib, gpu, shape):
+    """B of 96 MB or more: from M = 6 the split-K kernel runs, with B copied past the caches (non-temporal hint)."""
+    M, N, K = shape
+    assert hgemm_lib.auto_plan(M, N, K)["kernel"].startswith("split-K")
+    A = oracle.fill((M, K), 33, 1, oracle.NORMAL, 0.0, 1.0)
+    B = oracle.fill((N, K), 33, 2, oracle.NORMAL, 0.0, 0.02)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    _assert_close(oracle, first, oracle.hgemm(A, B), K)
+    assert np.array_equal(first, second)
+    At, Bt = oracle.fill((M, K), 34, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 34, 2, oracle.TERNARY, 0, 1)
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
