@@ -81,12 +81,12 @@ def _cpu_baseline(torch, A, B, C, budget_s=12.0):
 
 
 def _loaded_library(needle: str):
-    """Path of the shared object whose name contains `needle`, as mapped into this process.  PyTorch wheels carry
+    """Path of the shared object whose file name starts with `needle`, as mapped into this process.  PyTorch wheels carry
     their own libhipblaslt.so.1; imported first, that copy answers the comparator's dependency on the same soname, so
     the comparator of this process is not necessarily the system ROCm's (the C++ driver links that one)."""
     try:
         with open("/proc/self/maps") as f:
-            paths = {line.split()[-1] for line in f if needle in line.rsplit("/", 1)[-1].lower() and "/" in line}
+            paths = {line.split()[-1] for line in f if "/" in line and line.rsplit("/", 1)[-1].lower().startswith(needle)}
         return sorted(paths)[0] if paths else None
     except OSError:
         return None
@@ -179,7 +179,7 @@ def main():
         "settle": {"what": "hipBLASLt launches of the same shape before the first timed leg", "calls": settle_calls,
                    "ms": settle_ms},
         "second_pass_tflops": lib.tflops(M, N, K, ms2),
-        "vendor": {"library": "hipBLASLt (fp32 compute)", "loaded_from": _loaded_library("hipblaslt"),
+        "vendor": {"library": "hipBLASLt (fp32 compute)", "loaded_from": _loaded_library("libhipblaslt.so"),
                    "tflops": vendor_tflops, "ms": min(vms, vms2),
                    "first_pass_tflops": lib.tflops(M, N, K, vms), "second_pass_tflops": lib.tflops(M, N, K, vms2),
                    "ours_over_vendor": tflops / vendor_tflops},
