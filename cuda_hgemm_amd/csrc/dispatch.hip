@@ -1,6 +1,7 @@
 // hgemm_skinny and hgemm_auto: shape-driven choice among the tuned kernels.
 #include "../../include/hgemm.h"
 #include "mfma_decode.h"
+#include "mfma_decode_ring.h"
 #include "mfma_pipelined.h"
 #include "mfma_ragged.h"
 #include "mfma_skinny.h"
@@ -313,6 +314,18 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     // a few rows: one streaming pass over B, no second launch; against a B of 96 MB or more the split-K kernel with
     // B streamed past the caches is ahead from M = 6 (N = 14336: 8-16 %, N = 28672: 2-3 %; K = 4096)
     const bool large_b = N * K >= ((size_t)48 << 20);
+    // M <= 16: the decode kernel with per-wave LDS rings, wherever it was measured ahead of the kernels below (K = 1024
+    // ... 28672 against N = 256 ... 28672, HBM-cold: 0-60 %, median 18 %).  Up to M = 8 that is everywhere except
+    // against a B of 96 MB or more with K < 8192 (ties) or K a multiple of 16384 (its 16 rows of B per workgroup then
+    // lie 32 KB apart: 20-28 % behind), and K < 2048 against N > 8192 (up to 4 % behind at M = 1).  Above M = 8 K slices
+    // across workgroups win from K = 5120 on unless N is small, and for N > 8192 or K >= 4 N.
+    const bool ring_small = !(large_b && (K < 8192 || K % 16384 == 0)) && !(K < 2048 && N > 8192);
+    const bool ring_mid = N <= 8192 && K < 4 * N && (K <= 4096 || (K <= 8192 && N <= 4096));
+    if (M <= 16 && decode_ring_supports(M, N, K) && K >= 1024 && (M <= 8 ? ring_small : ring_mid)) {
+        p.kernel = KERNEL_DECODE_RING;
+        p.splits = decode_ring_waves(N, K, cus);
+        return p;
+    }
     if (M <= 8 && decode_supports(M, N, K) && !(M >= 6 && large_b && skinny_supports(M, N, K))) {
         int bn = 16, waves = 1;
         decode_plan(M, N, K, cus, &bn, &waves);
@@ -533,6 +546,7 @@ void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, 
         case KERNEL_SPLIT_128x128: launch_splitk<Split128x128>(A, B, C, M, N, K, p.splits, ws); break;
         case KERNEL_DECODE_BN16: launch_decode(A, B, C, M, N, K, 16, p.splits); break;
         case KERNEL_DECODE_BN32: launch_decode(A, B, C, M, N, K, 32, p.splits); break;
+        case KERNEL_DECODE_RING: launch_decode_ring(A, B, C, M, N, K, p.splits); break;
         case KERNEL_RAGGED: launch_ragged(A, B, C, M, N, K); break;
         case KERNEL_PADDED: run_padded(p, ws, A, B, C, M, N, K); break;
         case KERNEL_SIMT:
@@ -715,6 +729,7 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
         case KERNEL_SPLIT_128x128: return "split-K 128x128x64, 4 waves, 4-stage ring";
         case KERNEL_DECODE_BN16: return "streaming decode, 16 columns per workgroup, one wave per K slice";
         case KERNEL_DECODE_BN32: return "streaming decode, 32 columns per workgroup, one wave per K slice";
+        case KERNEL_DECODE_RING: return "streaming decode, 16 columns per workgroup, one wave and one LDS ring per K slice";
         case KERNEL_RAGGED: return "guarded 128x128x32, 4 waves, any shape";
         case KERNEL_PADDED: return "zero-padded operand copies + pipelined kernel of the padded shape";
         case KERNEL_SIMT: return "scalar fallback";

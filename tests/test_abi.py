@@ -103,6 +103,9 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
             p = plan(m, n, 4096)
             if m <= 8 and not (m >= 6 and n == 28672):     # from M = 6 a B of 96 MB or more goes to the split-K kernel
                 assert p["kernel"].startswith("streaming decode"), (m, n, p)
+                assert ("LDS ring" in p["kernel"]) == (n == 4096), (m, n, p)
+            elif m == 16 and n == 4096:                     # up to M = 16 the decode kernel with per-wave LDS rings
+                assert "LDS ring" in p["kernel"] and p["splits"] == 4, (m, n, p)
             else:
                 assert p["kernel"].startswith("split-K"), (m, n, p)
             assert 4096 % (p["splits"] * 64) == 0

@@ -371,6 +371,25 @@ def test_streaming_decode_kernel(oracle, hgemm_lib, gpu, shape):
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
+@pytest.mark.parametrize("shape", [(1, 4096, 4096), (16, 4096, 4096), (9, 272, 1024), (13, 1040, 1152), (16, 8192, 1024),
+                                   (3, 16, 3072), (8, 2048, 8192), (11, 4096, 8192), (16, 336, 1280), (2, 14336, 2048),
+                                   (5, 8192, 8192), (7, 4112, 16384 - 128)])
+def test_decode_kernel_with_lds_rings(oracle, hgemm_lib, gpu, shape):
+    """M <= 16 through per-wave LDS rings: two, four and eight K slices per workgroup, slices of one chunk and of
+    many (127 when only two waves divide K), slices shorter than the ring, N of one to 896 column tiles, rows of A
+    beyond M."""
+    M, N, K = shape
+    plan = hgemm_lib.auto_plan(M, N, K)
+    assert "LDS ring" in plan["kernel"] and K % (plan["splits"] * 64) == 0, plan
+    A = oracle.fill((M, K), 35, 1, oracle.NORMAL, 0.0, 1.0)
+    B = oracle.fill((N, K), 35, 2, oracle.NORMAL, 0.0, 0.02)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    _assert_close(oracle, first, oracle.hgemm(A, B), K)
+    assert np.array_equal(first, second)
+    At, Bt = oracle.fill((M, K), 36, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 36, 2, oracle.TERNARY, 0, 1)
+    assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
+
+
 @pytest.mark.parametrize("shape", [(7, 28672, 2048), (8, 20480, 2816), (6, 14336, 4096), (100, 14336, 4096)])
 def test_small_m_against_a_large_b(oracle, hgemm_lib, gpu, shape):
     """B of 96 MB or more: from M = 6 the split-K kernel runs, with B copied past the caches (non-temporal hint)."""
