@@ -314,16 +314,21 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     // a few rows: one streaming pass over B, no second launch; against a B of 96 MB or more the split-K kernel with
     // B streamed past the caches is ahead from M = 6 (N = 14336: 8-16 %, N = 28672: 2-3 %; K = 4096)
     const bool large_b = N * K >= ((size_t)48 << 20);
-    // M <= 16: the decode kernel with per-wave LDS rings, wherever it was measured ahead of the kernels below (K = 1024
+    // M <= 64: the decode kernel with per-wave LDS rings, wherever it was measured ahead of the kernels below (K = 1024
     // ... 28672 against N = 256 ... 28672, HBM-cold: 0-60 %, median 18 %).  Up to M = 8 that is everywhere except
     // against a B of 96 MB or more with K < 8192 (ties) or K a multiple of 16384 (its 16 rows of B per workgroup then
     // lie 32 KB apart: 20-28 % behind), and K < 2048 against N > 8192 (up to 4 % behind at M = 1).  Above M = 8 K slices
     // across workgroups win from K = 5120 on unless N is small, and for N > 8192 or K >= 4 N.
     const bool ring_small = !(large_b && (K < 8192 || K % 16384 == 0)) && !(K < 2048 && N > 8192);
     const bool ring_mid = N <= 8192 && K < 4 * N && (K <= 4096 || (K <= 8192 && N <= 4096));
-    if (M <= 16 && decode_ring_supports(M, N, K) && K >= 1024 && (M <= 8 ? ring_small : ring_mid)) {
+    // M = 17 ... 64 (two or four row tiles of A per wave): while K is short, where one launch beats the split-K kernel
+    // and the launch that adds its slices.  Old library against new, K = 1024 ... 4096 against N = 272 ... 8192: ahead
+    // by 0-126 % (median 31 %, 180 shapes) for K <= 2048 up to N = 4096; beyond that mixed (M = 32: 15 % behind to 6 % ahead).
+    const bool ring_tall = K < 4 * N && N <= 4096 && K <= 2048;
+    if (M <= 64 && decode_ring_supports(M, N, K) && K >= 1024 &&
+        (M <= 8 ? ring_small : M <= 16 ? ring_mid : ring_tall)) {
         p.kernel = KERNEL_DECODE_RING;
-        p.splits = decode_ring_waves(N, K, cus);
+        p.splits = decode_ring_waves(M, N, K, cus);
         return p;
     }
     if (M <= 8 && decode_supports(M, N, K) && !(M >= 6 && large_b && skinny_supports(M, N, K))) {
