@@ -324,8 +324,10 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     // M = 17 ... 64 (two or four row tiles of A per wave): while K is short, where one launch beats the split-K kernel
     // and the launch that adds its slices.  Old library against new, K = 1024 ... 4096 against N = 272 ... 8192: ahead
     // by 0-126 % (median 31 %, 180 shapes) for K <= 2048 up to N = 4096; beyond that mixed (M = 32: 15 % behind to 6 % ahead).
-    const bool ring_tall = K < 4 * N && N <= 4096 && K <= 2048;
-    if (M <= 64 && decode_ring_supports(M, N, K) && K >= 1024 &&
+    const bool ring_tall = K < 4 * N && N <= (K < 1024 ? 8192u : 4096u) && K <= 2048;
+    // K < 1024: up to M = 8 the streaming kernel is as fast or faster (one launch too); above, the same comparison
+    // (K = 256 ... 896 against N = 272 ... 8192) has the ring kernel ahead throughout
+    if (M <= 64 && decode_ring_supports(M, N, K) && K >= (M <= 8 ? 1024u : 256u) &&
         (M <= 8 ? ring_small : M <= 16 ? ring_mid : ring_tall)) {
         p.kernel = KERNEL_DECODE_RING;
         p.splits = decode_ring_waves(M, N, K, cus);
