@@ -314,7 +314,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     // a few rows: one streaming pass over B, no second launch; against a B of 96 MB or more the split-K kernel with
     // B streamed past the caches is ahead from M = 6 (N = 14336: 8-16 %, N = 28672: 2-3 %; K = 4096)
     const bool large_b = N * K >= ((size_t)48 << 20);
-    // M <= 64: the decode kernel with per-wave LDS rings, wherever it was measured ahead of the kernels below (K = 1024
+    // M <= 128: the decode kernel with per-wave LDS rings, wherever it was measured ahead of the kernels below (K = 1024
     // ... 28672 against N = 256 ... 28672, HBM-cold: 0-60 %, median 18 %).  Up to M = 8 that is everywhere except
     // against a B of 96 MB or more with K < 8192 (ties) or K a multiple of 16384 (its 16 rows of B per workgroup then
     // lie 32 KB apart: 20-28 % behind), and K < 2048 against N > 8192 (up to 4 % behind at M = 1).  Above M = 8 K slices
@@ -327,8 +327,10 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     const bool ring_tall = K < 4 * N && N <= (K < 1024 ? 8192u : 4096u) && K <= 2048;
     // K < 1024: up to M = 8 the streaming kernel is as fast or faster (one launch too); above, the same comparison
     // (K = 256 ... 896 against N = 272 ... 8192) has the ring kernel ahead throughout
-    if (M <= 64 && decode_ring_supports(M, N, K) && K >= (M <= 8 ? 1024u : 256u) &&
-        (M <= 8 ? ring_small : M <= 16 ? ring_mid : ring_tall)) {
+    // M = 65 ... 128 (eight row tiles): K <= 1024 up to N = 4096, K <= 512 up to N = 8192 (15-100 % ahead)
+    const bool ring_tallest = K < 4 * N && K <= 1024 && N <= (K <= 512 ? 8192u : 4096u);
+    if (M <= 128 && decode_ring_supports(M, N, K) && K >= (M <= 8 ? 1024u : 256u) &&
+        (M <= 8 ? ring_small : M <= 16 ? ring_mid : M <= 64 ? ring_tall : ring_tallest)) {
         p.kernel = KERNEL_DECODE_RING;
         p.splits = decode_ring_waves(M, N, K, cus);
         return p;

@@ -1,4 +1,4 @@
-// Decode-shaped product, M <= 64, through per-wave LDS rings.
+// Decode-shaped product, M <= 128, through per-wave LDS rings.
 //
 // Like the streaming decode kernel, a workgroup owns 16 rows of B (16 columns of C), each of
 // its waves owns one slice of K, there is no barrier in the loop and the waves add their fp32
@@ -12,9 +12,10 @@
 // cover eight rows x 128 contiguous bytes per instruction, into a ring of its own, and reads
 // the operands back with ds_read_b128.  The ring belongs to one wave, so the only
 // synchronisation is the wave's own vmcnt wait (copies complete in order) and an lgkmcnt(0)
-// before a slot is refilled.  N = K = 4096: 7.6 / 8.0 / 8.3 us for M = 1 / 8 / 16.  With two or
-// four 16-row tiles of A per wave (M <= 32, 64) the kernel still saves the split-K kernel's
-// second launch, which pays while K is short (K = 1024, N = 4096, M = 32: 8.3 -> 4.8 us).
+// before a slot is refilled.  N = K = 4096: 7.6 / 8.0 / 8.3 us for M = 1 / 8 / 16.  With two,
+// four or eight 16-row tiles of A per wave (M <= 32, 64, 128) the kernel still saves the
+// split-K kernel's second launch, which pays while K is short (K = 1024, N = 4096, M = 32:
+// 8.3 -> 4.8 us; K = 512, N = 4096, M = 128: 10.8 -> 5.9 us).
 //
 // LDS layout of one chunk: 16 TM rows x 128 bytes of A, then 16 rows of B.  A direct-to-LDS
 // load writes lane l's 16 bytes at byte 16 * l of a 1 KB block, so block h holds rows
@@ -139,9 +140,9 @@ __global__ void __launch_bounds__(RING_MAX_WAVES * 64)
     }
 }
 
-// M <= 64, N a multiple of 16, K a multiple of 128 (two waves get whole 64-wide chunks).
+// M <= 128, N a multiple of 16, K a multiple of 128 (two waves get whole 64-wide chunks).
 inline bool decode_ring_supports(size_t M, size_t N, size_t K) {
-    return M >= 1 && M <= 64 && N > 0 && N % 16 == 0 && K > 0 && K % 128 == 0 && N <= ((size_t)1 << 31) / 16;
+    return M >= 1 && M <= 128 && N > 0 && N % 16 == 0 && K > 0 && K % 128 == 0 && N <= ((size_t)1 << 31) / 16;
 }
 
 inline int decode_ring_max_waves(size_t M);
@@ -150,6 +151,7 @@ inline int decode_ring_max_waves(size_t M);
 // so they stream from HBM): a wave should own 640 ... 1280 of K (eight waves' rings leave room for one workgroup per
 // CU, four waves' for two), but there should be four waves unless N alone provides two or more workgroups per CU.
 inline int decode_ring_waves(size_t M, size_t N, size_t K, size_t cus) {
+    if (M > 64) return N / 16 <= cus ? 2 : 1;  // eight row tiles of A: two waves only while N gives one workgroup per CU
     int w = 2;
     while (w < decode_ring_max_waves(M) && K / (size_t)w > 1280) w *= 2;
     if (w < 4 && N / 16 < 2 * cus) w = 4;
@@ -174,21 +176,23 @@ void launch_decode_ring_tile(const void *A, const void *B, void *C, size_t M, si
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 
-// Rings of four chunks for one or two row tiles of A (16 and 24 KB per wave), of three for four (30 KB): up to eight,
-// four and four waves fit the 160 KB of a CU.
-inline int decode_ring_max_waves(size_t M) { return M <= 16 ? RING_MAX_WAVES : 4; }
+// Rings of four chunks for one or two row tiles of A (16 and 24 KB per wave), of three for four and eight (30 and
+// 54 KB): up to eight, four, four and two waves fit the 160 KB of a CU.
+inline int decode_ring_max_waves(size_t M) { return M <= 16 ? RING_MAX_WAVES : M <= 64 ? 4 : 2; }
 
 inline void launch_decode_ring(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, int waves) {
     check_operands(A, B, C, M, N, K);
-    HGEMM_CHECK_MSG(decode_ring_supports(M, N, K), "ring decode kernel needs M <= 64, N %% 16 == 0, K %% 128 == 0 (got M=%zu N=%zu K=%zu)",
+    HGEMM_CHECK_MSG(decode_ring_supports(M, N, K), "ring decode kernel needs M <= 128, N %% 16 == 0, K %% 128 == 0 (got M=%zu N=%zu K=%zu)",
                     M, N, K);
     HGEMM_CHECK(waves >= 1 && waves <= decode_ring_max_waves(M) && K % ((size_t)waves * 64) == 0);
     if (M <= 16)
         launch_decode_ring_tile<1, 4>(A, B, C, M, N, K, waves);
     else if (M <= 32)
         launch_decode_ring_tile<2, 4>(A, B, C, M, N, K, waves);
-    else
+    else if (M <= 64)
         launch_decode_ring_tile<4, 3>(A, B, C, M, N, K, waves);
+    else
+        launch_decode_ring_tile<8, 3>(A, B, C, M, N, K, waves);
 }
 
 }  // namespace hgemm

@@ -23,7 +23,7 @@ enum KernelId {
     KERNEL_DECODE_BN32,
     KERNEL_SMALL64_W4,  // 64x64x64 tile on four waves of 32x32 (the ladder's kernel): grids of at most one tile per CU
     KERNEL_MID128_S2,   // pipelined 128x128x64, 4 waves, 2-stage ring: two workgroups per CU, for K of at most four chunks
-    KERNEL_DECODE_RING, // decode kernel for M <= 64 whose waves stage operands through LDS rings of their own; `splits` waves over K
+    KERNEL_DECODE_RING, // decode kernel for M <= 128 whose waves stage operands through LDS rings of their own; `splits` waves over K
     KERNEL_PADDED,      // operands copied zero-padded to N % 8 == 0, K % 64 == 0, then the plan for that shape
 };
 
