@@ -103,9 +103,9 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
             p = plan(m, n, 4096)
             if m <= 8 and not (m >= 6 and n == 28672):     # from M = 6 a B of 96 MB or more goes to the split-K kernel
                 assert p["kernel"].startswith("streaming decode"), (m, n, p)
-                assert ("LDS ring" in p["kernel"]) == (n == 4096), (m, n, p)
+                assert ("LDS ring per K slice" in p["kernel"]) == (n == 4096), (m, n, p)
             elif m == 16 and n == 4096:                     # up to M = 16 the decode kernel with per-wave LDS rings
-                assert "LDS ring" in p["kernel"] and p["splits"] == 4, (m, n, p)
+                assert "LDS ring per K slice" in p["kernel"] and p["splits"] == 4, (m, n, p)
             else:
                 assert p["kernel"].startswith("split-K"), (m, n, p)
             assert 4096 % (p["splits"] * 64) == 0
@@ -124,6 +124,8 @@ def test_auto_plan_invariants_over_many_shapes(hgemm_lib):
     shapes = [(t, t, k) for t in range(64, 3073, 64) for k in (64, 128, 192, 256, 320, 1024, 2560, 4096, 16384)]
     for _ in range(1500):
         shapes.append((rng.randrange(1, 9000), 8 * rng.randrange(1, 1100), 64 * rng.randrange(1, 260)))
+    for _ in range(1500):                                                   # small M: the decode and split-K kernels
+        shapes.append((rng.randrange(1, 130), 16 * rng.randrange(1, 2000), 64 * rng.randrange(1, 300)))
     cus = 256
     for (m, n, k) in shapes:
         p = hgemm_lib.auto_plan(m, n, k)
@@ -141,6 +143,11 @@ def test_auto_plan_invariants_over_many_shapes(hgemm_lib):
                 assert s == 1 and k // 64 < 40, (m, n, k, p)
         if "2-stage ring" in p["kernel"]:
             assert k <= 256 and s == 1 and p["tail_tiles"] == 0, (m, n, k, p)
+        if "LDS ring per K slice" in p["kernel"]:
+            # whole 64-wide chunks per wave; the waves' rings (16, 24, 30, 54 KB for 1, 2, 4, 8 row tiles of A) fit a CU
+            assert m <= 128 and n % 16 == 0 and k % (64 * s) == 0 and need == {"partial": 0, "operands": 0}, (m, n, k, p)
+            ring_kb = 16 if m <= 16 else 24 if m <= 32 else 30 if m <= 64 else 54
+            assert s * ring_kb <= 160, (m, n, k, p)
 
 
 def test_workspace_needs_of_auto_plans(hgemm_lib):

@@ -383,7 +383,7 @@ def test_decode_kernel_with_lds_rings(oracle, hgemm_lib, gpu, shape):
     beyond M."""
     M, N, K = shape
     plan = hgemm_lib.auto_plan(M, N, K)
-    assert "LDS ring" in plan["kernel"] and K % (plan["splits"] * 64) == 0, plan
+    assert "LDS ring per K slice" in plan["kernel"] and K % (plan["splits"] * 64) == 0, plan
     A = oracle.fill((M, K), 35, 1, oracle.NORMAL, 0.0, 1.0)
     B = oracle.fill((N, K), 35, 2, oracle.NORMAL, 0.0, 0.02)
     first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
