@@ -15,7 +15,7 @@
 // before a slot is refilled.  N = K = 4096: 7.6 / 8.0 / 8.3 us for M = 1 / 8 / 16.  With two,
 // four or eight 16-row tiles of A per wave (M <= 32, 64, 128) the kernel still saves the
 // split-K kernel's second launch, which pays while K is short (K = 1024, N = 4096, M = 32:
-// 8.3 -> 4.8 us; K = 512, N = 4096, M = 128: 10.8 -> 5.9 us).
+// 6.5 -> 4.8 us; K = 512, N = 4096, M = 128: 11.0 -> 6.1 us).
 //
 // LDS layout of one chunk: 16 TM rows x 128 bytes of A, then 16 rows of B.  A direct-to-LDS
 // load writes lane l's 16 bytes at byte 16 * l of a 1 KB block, so block h holds rows
