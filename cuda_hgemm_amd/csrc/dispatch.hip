@@ -324,7 +324,8 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     // M = 17 ... 64 (two or four row tiles of A per wave): while K is short, where one launch beats the split-K kernel
     // and the launch that adds its slices.  Old library against new, K = 1024 ... 4096 against N = 272 ... 8192: ahead
     // by 0-126 % (median 31 %, 180 shapes) for K <= 2048 up to N = 4096; beyond that mixed (M = 32: 15 % behind to 6 % ahead).
-    const bool ring_tall = K < 4 * N && N <= (K < 1024 ? 8192u : 4096u) && K <= 2048;
+    // (and up to K = 4096 for M <= 24 against N = 3072 ... 4096: 13-40 % ahead; at N <= 2048 M = 24 is 1-9 % behind)
+    const bool ring_tall = K < 4 * N && N <= (K < 1024 ? 8192u : 4096u) && (K <= 2048 || (M <= 24 && N >= 3072 && K <= 4096));
     // K < 1024: up to M = 8 the streaming kernel is as fast or faster (one launch too); above, the same comparison
     // (K = 256 ... 896 against N = 272 ... 8192) has the ring kernel ahead throughout
     // M = 65 ... 128 (eight row tiles): K <= 1024 up to N = 4096, K <= 512 up to N = 8192 (15-100 % ahead)
