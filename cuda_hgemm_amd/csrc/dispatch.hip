@@ -330,7 +330,8 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     // (K = 256 ... 896 against N = 272 ... 8192) has the ring kernel ahead throughout
     // M = 65 ... 128 (eight row tiles): K <= 1024 up to N = 4096, K <= 512 up to N = 8192 (15-100 % ahead)
     const bool ring_tallest = K < 4 * N && K <= 1024 && N <= (K <= 512 ? 8192u : 4096u);
-    if (M <= 128 && decode_ring_supports(M, N, K) && K >= (M <= 8 ? 1024u : 256u) &&
+    // (M <= 8 below K = 1024 only where the streaming kernel cannot run: N % 32 or K % 256 nonzero)
+    if (M <= 128 && decode_ring_supports(M, N, K) && K >= (M <= 8 && decode_supports(M, N, K) ? 1024u : 256u) &&
         (M <= 8 ? ring_small : M <= 16 ? ring_mid : M <= 64 ? ring_tall : ring_tallest)) {
         p.kernel = KERNEL_DECODE_RING;
         p.splits = decode_ring_waves(M, N, K, cus);

@@ -376,7 +376,7 @@ def test_streaming_decode_kernel(oracle, hgemm_lib, gpu, shape):
                                    (5, 8192, 8192), (7, 4112, 16384 - 128), (17, 4096, 2048), (32, 4096, 1024),
                                    (24, 1040, 1280), (33, 4096, 2048), (64, 4096, 1024), (48, 2064, 1152), (40, 272, 1024),
                                    (16, 4096, 256), (64, 8192, 896), (33, 272, 384), (9, 1040, 640),
-                                   (65, 4096, 1024), (128, 8192, 512), (100, 272, 384), (128, 4096, 256), (24, 4096, 4096)])
+                                   (65, 4096, 1024), (128, 8192, 512), (100, 272, 384), (128, 4096, 256), (24, 4096, 4096), (5, 1040, 384), (8, 4096, 640)])
 def test_decode_kernel_with_lds_rings(oracle, hgemm_lib, gpu, shape):
     """M <= 128 through per-wave LDS rings (one, two, four or eight 16-row tiles of A per wave): one, two, four and eight K slices per workgroup, slices of one chunk and of
     many (127 when only two waves divide K), slices shorter than the ring, N of one to 896 column tiles, rows of A
