@@ -3,8 +3,6 @@
     cuda_hgemm_amd/lib/libhgemm.so            the kernels + C ABI (include/hgemm.h)
     cuda_hgemm_amd/lib/libhgemm_hipblaslt.so  vendor comparator (include/hgemm_hipblaslt.h)
     cuda_hgemm_amd/bin/hgemm                  C++ benchmark / check driver
-    cuda_hgemm_amd/bin/hgemm_probe            in-kernel timing of the tuned kernels (evidence tool)
-    cuda_hgemm_amd/bin/hgemm_mix_probe        cost of each piece of their loop under the power limit (evidence tool)
 
 Run as ``python -m cuda_hgemm_amd.build`` (add ``--force`` to rebuild everything).
 hipcc cross-compiles without a GPU, so this works on a CPU-only machine.
@@ -13,6 +11,7 @@ from __future__ import annotations
 
 import concurrent.futures as cf
 import os
+import re
 import subprocess
 import sys
 
@@ -34,9 +33,6 @@ LIB_SOURCES = ["basic_kernels.hip", "ladder_sync.hip", "ladder_async.hip", "ladd
                "api.hip"]
 VENDOR_SOURCES = ["vendor_hipblaslt.cpp"]
 DRIVER_SOURCES = ["driver/main.cpp"]
-# evidence tools, not part of the library: bin/hgemm_probe (in-kernel timing of the tuned kernels)
-# and bin/hgemm_mix_probe (what each piece of their loop costs under the power limit)
-PROBE_SOURCES = ["probe/probe_loop.hip", "probe/issue_mix.hip"]
 
 
 def _headers():
@@ -64,28 +60,63 @@ def _run(cmd):
 
 # Kernels whose operands and accumulators are handled from inline assembly in an order the
 # compiler does not know: a register spill between an LDS read and its wait, or of an
-# accumulator, would corrupt results silently, and the chained kernel keeps its accumulators
-# in AGPRs the compiler must never look for, so the build fails if a spill appears.
+# accumulator, would corrupt results silently, so the build fails if one appears.  The chained
+# kernel keeps its accumulators in AGPRs a0 ... a(4*TM*TN-1) that only its asm statements name:
+# it must use exactly that many AGPRs (one more would be an accumulator register the compiler
+# took for itself) and fewer than 256 VGPRs (beyond them the allocator starts looking for AGPRs).
 NO_SPILL_KERNELS = ("hgemm_pipelined_kernel", "hgemm_chained_kernel")
+# sources that must contain such kernels: a remark format the parser no longer understands
+# must not turn the guard into a no-op
+MUST_CHECK = {"dispatch.hip": NO_SPILL_KERNELS}
+
+
+def _chained_accumulator_registers(mangled):
+    """4 * PTM * PTN of a hgemm_chained_kernel instantiation, from the PipeConfig arguments in
+    its mangled name (BM, BN, BK, WAVES_M, WAVES_N, STAGES, MI, ...): 16x16 tiles, 4 registers each."""
+    m = re.search(r"PipeConfigI((?:Li\d+E)+)E", mangled)
+    if not m:
+        raise RuntimeError(f"cannot read the tile configuration out of {mangled}")
+    bm, bn, _bk, waves_m, waves_n, _stages, mi = [int(v) for v in re.findall(r"Li(\d+)E", m.group(1))[:7]]
+    return 4 * (bm // waves_m // mi) * (bn // waves_n // mi)
 
 
 def _check_no_spills(src, remarks):
-    """`remarks`: output of -Rpass-analysis=kernel-resource-usage for one source file."""
-    name, checked = None, 0
+    """`remarks`: output of -Rpass-analysis=kernel-resource-usage for one source file.
+    Returns the names of the guarded kernel templates that were seen and checked."""
+    usage = {}  # kernel -> {key: value}
+    name = None
     for line in remarks.splitlines():
         if "remark: Function Name:" in line:
             name = line.split("Function Name:")[1].split()[0]
+            usage[name] = {}
             continue
-        if name is None or not any(k in name for k in NO_SPILL_KERNELS):
+        if name is None:
             continue
-        for key in ("ScratchSize [bytes/lane]:", "SGPRs Spill:", "VGPRs Spill:"):
-            if key in line:
-                value = int(line.split(key)[1].split()[0])
-                checked += 1
-                if value != 0 and key != "SGPRs Spill:":
-                    raise RuntimeError(f"{src}: kernel {name} has {key} {value}; its inline-assembly schedule "
-                                       "needs every operand and accumulator in registers")
-    return checked
+        for key in ("ScratchSize [bytes/lane]:", "VGPRs Spill:", "VGPRs:", "AGPRs:"):
+            if "remark:     " + key in line or "remark: " + key in line:
+                usage[name][key] = int(line.split(key)[1].split()[0])
+    seen = set()
+    for name, u in usage.items():
+        kind = next((k for k in NO_SPILL_KERNELS if k in name), None)
+        if kind is None:
+            continue
+        missing = [k for k in ("ScratchSize [bytes/lane]:", "VGPRs Spill:", "VGPRs:", "AGPRs:") if k not in u]
+        if missing:
+            raise RuntimeError(f"{src}: no {missing} remark for kernel {name}: the resource guard cannot check it")
+        for key in ("ScratchSize [bytes/lane]:", "VGPRs Spill:"):
+            if u[key] != 0:
+                raise RuntimeError(f"{src}: kernel {name} has {key} {u[key]}; its inline-assembly schedule "
+                                   "needs every operand and accumulator in registers")
+        if kind == "hgemm_chained_kernel":
+            want = _chained_accumulator_registers(name)
+            if u["AGPRs:"] != want or u["VGPRs:"] >= 256:
+                raise RuntimeError(f"{src}: kernel {name} uses {u['AGPRs:']} AGPRs and {u['VGPRs:']} VGPRs; its named "
+                                   f"accumulators need exactly {want} AGPRs and fewer than 256 VGPRs")
+        seen.add(kind)
+    for kind in MUST_CHECK.get(os.path.basename(src), ()):
+        if kind not in seen:
+            raise RuntimeError(f"{src}: the resource guard found no {kind} in the compiler's remarks")
+    return seen
 
 
 def _compile(src, force):
@@ -93,7 +124,7 @@ def _compile(src, force):
     path = os.path.join(CSRC, src)
     if force or _stale(obj, [path] + _headers()):
         flags = CXXFLAGS + (DEVICE_FLAGS if src.endswith(".hip") else [])
-        if src.startswith("driver/") or src.startswith("probe/"):
+        if src.startswith("driver/"):
             flags = flags + ["-fopenmp"]
         if src.endswith(".hip"):
             flags = flags + ["-Rpass-analysis=kernel-resource-usage"]
@@ -110,7 +141,7 @@ def _compile(src, force):
 def build(force: bool = False, verbose: bool = False) -> dict:
     for d in (OBJ, LIB, BIN):
         os.makedirs(d, exist_ok=True)
-    sources = LIB_SOURCES + VENDOR_SOURCES + DRIVER_SOURCES + PROBE_SOURCES
+    sources = LIB_SOURCES + VENDOR_SOURCES + DRIVER_SOURCES
     with cf.ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
         objs = dict(zip(sources, pool.map(lambda s: _compile(s, force), sources)))
     libhgemm = os.path.join(LIB, "libhgemm.so")
@@ -126,14 +157,9 @@ def build(force: bool = False, verbose: bool = False) -> dict:
     if force or _stale(driver, drv_objs + [libhgemm, vendor]):
         _run([HIPCC, "-o", driver] + drv_objs + ["-L" + LIB, "-lhgemm", "-lhgemm_hipblaslt", "-fopenmp",
                                                   "-Wl,-rpath,$ORIGIN/../lib"])
-    probes = {}
-    for src, name in zip(PROBE_SOURCES, ("hgemm_probe", "hgemm_mix_probe")):
-        probes[name] = os.path.join(BIN, name)
-        if force or _stale(probes[name], [objs[src]]):
-            _run([HIPCC, "-o", probes[name], objs[src], "-fopenmp"])
     if verbose:
-        print("built", libhgemm, vendor, driver, *probes.values())
-    return {"libhgemm": libhgemm, "vendor": vendor, "driver": driver, **probes}
+        print("built", libhgemm, vendor, driver)
+    return {"libhgemm": libhgemm, "vendor": vendor, "driver": driver}
 
 
 if __name__ == "__main__":

@@ -27,42 +27,61 @@ int current_device() {
 // Heap workspaces of hgemm_auto / hgemm_skinny, one pair per device, kept for the life of
 // the process (the reference keeps its vendor handle the same way,
 // src/cublas_tensor_op.cu:18).  Each is allocated once, at its cap, the first time a plan
-// needs it (or by hgemm_reserve_workspace), so a later call with a larger shape never
-// reallocates: no hipFree, no device synchronisation inside an entry point.  If the cap
-// cannot be had, the size asked for is tried; if that fails too the caller plans again
-// without a workspace.
+// needs it (or by hgemm_reserve_workspace).  If the cap cannot be had, the size asked for is
+// tried, and sizes hipMalloc has refused are remembered so that no later call asks again.
+// An entry point never frees or replaces a buffer: a plan that needs more than the buffer
+// holds (possible only after such a refusal) is not run, the caller plans again without a
+// workspace.  Only hgemm_reserve_workspace and hgemm_release_workspace replace or free, after
+// waiting for the device.
+//
+// g_heap_mutex guards the table AND is held while the launches of a plan that uses a
+// workspace are enqueued: every launch goes to the null stream, which runs them in the order
+// they were enqueued, so with the lock held two host threads cannot interleave one plan's
+// partial-sum kernel with the other's reduction, and no thread holds a workspace pointer
+// while another frees it.
+struct HeapState {
+    Workspace ws;
+    size_t partial_refused = SIZE_MAX, operand_refused = SIZE_MAX;  // smallest size hipMalloc has refused
+};
 std::mutex g_heap_mutex;
-Workspace g_heap[MAX_DEVICES];
+HeapState g_heap[MAX_DEVICES];
 
-bool grow(void **ptr, size_t *have, size_t need, size_t cap) {
+// Caller holds g_heap_mutex.  `may_replace`: an existing, smaller buffer may be freed (after a device synchronisation).
+bool grow(void **ptr, size_t *have, size_t need, size_t cap, size_t *refused, bool may_replace) {
     if (need <= *have) return true;
-    if (*ptr) {  // only hgemm_reserve_workspace can ask for more than the cap that was allocated
+    if (need >= *refused) return false;
+    if (*ptr) {
+        if (!may_replace) return false;
         HGEMM_CHECK_HIP_ERROR(hipDeviceSynchronize());
         HGEMM_CHECK_HIP_ERROR(hipFree(*ptr));
         *ptr = nullptr;
         *have = 0;
     }
     for (size_t want : {need > cap ? need : cap, need}) {
+        if (want >= *refused) continue;
         if (hipMalloc(ptr, want) == hipSuccess) {
             *have = want;
             return true;
         }
         (void)hipGetLastError();  // clear the allocation failure
         *ptr = nullptr;
+        *refused = want;
     }
     return false;
 }
 
-// The device's heap workspace with at least the given sizes; false if memory ran out.
-bool heap_workspace(size_t partial_bytes, size_t operand_bytes, Workspace *out) {
-    const int dev = current_device();
-    std::lock_guard<std::mutex> lock(g_heap_mutex);
-    Workspace &w = g_heap[dev];
+// The device's heap workspace with at least the given sizes; false if it does not hold them and
+// cannot be made to.  Caller holds g_heap_mutex.
+bool heap_workspace(size_t partial_bytes, size_t operand_bytes, Workspace *out, bool may_replace) {
+    HeapState &h = g_heap[current_device()];
+    Workspace &w = h.ws;
     bool ok = true;
     if (partial_bytes > w.partial_bytes)
-        ok = grow(reinterpret_cast<void **>(&w.partial), &w.partial_bytes, partial_bytes, MAX_PARTIAL_BYTES) && ok;
+        ok = grow(reinterpret_cast<void **>(&w.partial), &w.partial_bytes, partial_bytes, MAX_PARTIAL_BYTES,
+                  &h.partial_refused, may_replace) && ok;
     if (operand_bytes > w.operand_bytes)
-        ok = grow(reinterpret_cast<void **>(&w.operands), &w.operand_bytes, operand_bytes, MAX_PADDED_BYTES) && ok;
+        ok = grow(reinterpret_cast<void **>(&w.operands), &w.operand_bytes, operand_bytes, MAX_PADDED_BYTES,
+                  &h.operand_refused, may_replace) && ok;
     *out = w;
     return ok;
 }
@@ -138,7 +157,7 @@ using Split128x64 = SkinnyConfig<128, 64, 2, 2, 4>;
 using Split128x128 = SkinnyConfig<128, 128, 2, 2, 4>;
 
 // 256x256x64 tile on v_mfma_f32_16x16x32_f16, two B buffers and three A buffers (all 160 KB of LDS)
-using Big256 = PipeConfig<256, 256, 64, 2, 2, 2, 16, 0, 1>;
+using Big256 = PipeConfig<256, 256, 64, 2, 2, 2, 16, 1>;
 using Mid128 = PipeConfig<128, 128, 64, 2, 2, 5, 16>;
 // two LDS buffers (64 KB): two workgroups fit a CU, and one's C tile goes out while the other multiplies.  Pays where
 // a workgroup's K loop is shorter than its epilogue and C outgrows the Infinity Cache: 16384^2 x 256 201 -> 170 us.
@@ -576,39 +595,45 @@ namespace {
 
 // Plans of the shapes this thread saw last: a 5 us launch should not re-run the cost model
 // (five tiles x K slices x tails, in doubles) on every call.  Direct-mapped, fixed size,
-// per thread: no allocation, no lock.
+// per thread: no allocation, no lock.  Two tables: the best plan, and the best plan that
+// needs no workspace (what runs when device memory for the workspace cannot be had).
 struct CachedPlan {
     size_t M = 0, N = 0, K = 0;
     Plan plan;
 };
 constexpr int PLAN_CACHE_SLOTS = 64;
 
-const Plan &cached_plan(size_t M, size_t N, size_t K) {
-    static thread_local CachedPlan cache[PLAN_CACHE_SLOTS];
+const Plan &cached_plan(size_t M, size_t N, size_t K, bool without_workspace = false) {
+    static thread_local CachedPlan cache[2][PLAN_CACHE_SLOTS];
     const size_t h = (M * 0x9e3779b97f4a7c15ull) ^ (N * 0xc2b2ae3d27d4eb4full) ^ (K * 0x165667b19e3779f9ull);
-    CachedPlan &slot = cache[(h >> 32) % PLAN_CACHE_SLOTS];
+    CachedPlan &slot = cache[without_workspace ? 1 : 0][(h >> 32) % PLAN_CACHE_SLOTS];
     if (slot.M != M || slot.N != N || slot.K != K) {
-        slot.plan = plan_for(M, N, K);
+        PlanLimits limits;
+        if (without_workspace) limits.partial_bytes = limits.operand_bytes = 0;
+        slot.plan = plan_for(M, N, K, limits);
         slot.M = M, slot.N = N, slot.K = K;
     }
     return slot.plan;
 }
 
-// Runs the cached plan of the shape on the heap workspace; when device memory for the
-// workspace cannot be had, the best plan that needs none (no K slices, the guarded kernel
-// instead of padded copies).
+// Runs the cached plan of the shape on the heap workspace; when the workspace does not hold
+// what the plan needs and device memory for it cannot be had, the best plan that needs none
+// (no K slices, the guarded kernel instead of padded copies).
 void run_with_heap_workspace(const void *A, const void *B, void *C, size_t M, size_t N, size_t K) {
     const Plan &p = cached_plan(M, N, K);
-    Workspace ws;
     if (p.partial_bytes == 0 && p.operand_bytes == 0) {
-        run_plan(p, ws, A, B, C, M, N, K);
-    } else if (heap_workspace(p.partial_bytes, p.operand_bytes, &ws)) {
-        run_plan(p, ws, A, B, C, M, N, K);
-    } else {
-        PlanLimits none;
-        none.partial_bytes = none.operand_bytes = 0;
-        run_plan(plan_for(M, N, K, none), Workspace(), A, B, C, M, N, K);
+        run_plan(p, Workspace(), A, B, C, M, N, K);
+        return;
     }
+    {
+        std::lock_guard<std::mutex> lock(g_heap_mutex);  // held while the plan's launches are enqueued
+        Workspace ws;
+        if (heap_workspace(p.partial_bytes, p.operand_bytes, &ws, false)) {
+            run_plan(p, ws, A, B, C, M, N, K);
+            return;
+        }
+    }
+    run_plan(cached_plan(M, N, K, true), Workspace(), A, B, C, M, N, K);
 }
 
 }  // namespace
@@ -630,7 +655,7 @@ extern "C" void hgemm_auto(const hgemm_half *A, const hgemm_half *B, hgemm_half 
 #define HGEMM_DEFINE_PIPELINED_VARIANT(symbol, Cfg, which)                                                   \
     extern "C" void symbol(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N,      \
                            size_t K) {                                                                       \
-        launch_pipelined<Cfg>(A, B, C, M, N, K, #symbol, nullptr, which);                                    \
+        launch_pipelined<Cfg>(A, B, C, M, N, K, #symbol, which);                                             \
     }                                                                                                        \
     extern "C" int symbol##_supports(size_t M, size_t N, size_t K) {                                         \
         return pipelined_supports_edges<Cfg>(M, N, K) ? 1 : 0;                                               \
@@ -646,18 +671,19 @@ HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_chained_256x128, Rect256x128, PipeKern
 HGEMM_DEFINE_PIPELINED_VARIANT(hgemm_mfma_chained_256x256, Big256, PipeKernel::Chained)
 
 extern "C" int hgemm_reserve_workspace(size_t partial_bytes, size_t operand_bytes) {
+    std::lock_guard<std::mutex> lock(g_heap_mutex);
     Workspace ws;
-    return heap_workspace(partial_bytes, operand_bytes, &ws) ? 0 : 1;
+    return heap_workspace(partial_bytes, operand_bytes, &ws, true) ? 0 : 1;
 }
 
 extern "C" void hgemm_release_workspace(void) {
     const int dev = current_device();
     std::lock_guard<std::mutex> lock(g_heap_mutex);
-    Workspace &w = g_heap[dev];
+    Workspace &w = g_heap[dev].ws;
     if (w.partial || w.operands) HGEMM_CHECK_HIP_ERROR(hipDeviceSynchronize());  // launches may still use them
     if (w.partial) HGEMM_CHECK_HIP_ERROR(hipFree(w.partial));
     if (w.operands) HGEMM_CHECK_HIP_ERROR(hipFree(w.operands));
-    w = Workspace();
+    g_heap[dev] = HeapState();
 }
 
 extern "C" int hgemm_auto_static_workspace(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N,
@@ -681,7 +707,12 @@ extern "C" int hgemm_auto_static_workspace(const hgemm_half *A, const hgemm_half
     }
     // Nothing in the array has to start at zero: every kernel that reads partial sums or padded
     // operands reads only what a kernel launched before it in this call has written in full.
-    run_plan(p, ws, A, B, C, M, N, K);
+    if (partial_bytes + p.operand_bytes > 0) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);  // one plan's launches at a time into the null stream
+        run_plan(p, ws, A, B, C, M, N, K);
+    } else {
+        run_plan(p, ws, A, B, C, M, N, K);
+    }
     return 0;
 }
 

@@ -114,108 +114,32 @@ __device__ __forceinline__ void store_chained_tile(unsigned char *lds, half_t *_
     });
 }
 
-// EDGE: M and N need not be multiples of the tile (N % 8 == 0 still, for aligned rows of
-// C).  Copies of rows beyond the matrix are redirected to its last row -- valid memory,
-// products never stored -- which costs nothing inside the loop; only the stores are guarded.
+// Tile, K slice, copy offsets and operand addresses come from PipeFrame (mfma_pipelined.h), as in the interleaved
+// kernel; EDGE as there.
 template <class Cfg, bool SPLIT = false, bool EDGE = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_chained_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
                            float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n,
-                           int first_block, int tail_tiles, int subdiv, long long *probe_out) {
+                           int first_block, int tail_tiles, int subdiv) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
-    constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS, CPR = Cfg::CPR, CPS = Cfg::CPS;
-    constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES, SA = Cfg::SA, SB = Cfg::SB;
+    constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS;
+    constexpr int SA = Cfg::SA, SB = Cfg::SB;
     constexpr int A_BYTES = Cfg::A_BYTES, B_BYTES = Cfg::B_BYTES, B_REGION = SA * A_BYTES;
     constexpr int A_DMA = Cfg::A_DMA, B_DMA = Cfg::B_DMA, L = A_DMA + B_DMA;
     constexpr int NFRAG = TM + TN, NMMA = TM * TN;
     static_assert(NFRAG <= NMMA, "at most one operand read is issued per MFMA slot");
     static_assert(MI == 16 && TM * TN <= 64, "the schedule and the named accumulator registers are laid out for 16x16x32 tiles");
-    long long t_begin = 0, t_loop = 0, t_epi = 0, c_loop = 0, c_epi = 0;
-    if constexpr (Cfg::TIMESTAMPS) t_begin = wall_clock64();
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
-
-    int tile_m, tile_n;
-    // the same in every launch that works on this problem (probe builds can force either order)
-    const bool blocked = (Cfg::DBG & 16) ? false : ((Cfg::DBG & 32) ? true : blocked_order(N, K));
-    // this workgroup's slot among the launch's positions: slots are dealt so that the workgroups an XCD runs
-    // together are neighbours in the tile order.  A K-sliced launch is one-dimensional as well, slice-major, so
-    // that those neighbours also work on the same slice of K.
-    int slot, slice = 0;
-    if constexpr (SPLIT) {
-        const int slices = K / k_len;
-        slice_and_slot_of_workgroup((int)blockIdx.x, (int)gridDim.x / slices, slices, slice, slot);
-        slice = __builtin_amdgcn_readfirstlane(slice);
-    } else {
-        slot = slot_of_workgroup(blocked, (int)blockIdx.x, (int)gridDim.x);
-    }
-    if (subdiv == 0) {
-        // the launch covers positions [first_block, first_block + gridDim.x) of the tile order
-        tile_of_position(blocked, first_block + slot, tiles_m, tiles_n, tile_m, tile_n);
-    } else {
-        // tiles_m x tiles_n is the grid of a larger tile that this one divides sub_m x sub_n times;
-        // consecutive slots take the parts of the tile at position first_block + slot / parts
-        const int sub_m = subdiv >> 8, sub_n = subdiv & 255, parts = sub_m * sub_n;
-        const int part = slot % parts;
-        int parent_m, parent_n;
-        tile_of_position(blocked, first_block + slot / parts, tiles_m, tiles_n, parent_m, parent_n);
-        tile_m = parent_m * sub_m + part / sub_n;
-        tile_n = parent_n * sub_n + part % sub_n;
-        if (tile_m * BM >= M || tile_n * BN >= N) return;  // a part wholly outside the matrix (whole workgroup)
-    }
-    tile_m = __builtin_amdgcn_readfirstlane(tile_m);  // wave-uniform by construction: keep them in SGPRs
-    tile_n = __builtin_amdgcn_readfirstlane(tile_n);
-    const int num_k = k_len / BK;
-    const int k_begin = slice * k_len;
-
-    // ---- copy set-up: wave w, instruction i fills LDS rows [(i*WAVES + w)*ROWS_PER_DMA, +ROWS_PER_DMA)
-    const unsigned char *a_base = reinterpret_cast<const unsigned char *>(A + (size_t)tile_m * BM * K + k_begin);
-    const unsigned char *b_base = reinterpret_cast<const unsigned char *>(B + (size_t)tile_n * BN * K + k_begin);
-    constexpr int DMA_ROW_STEP = Cfg::WAVES * Cfg::ROWS_PER_DMA;
-    uint32_t voff[L];
-    {
-        // lane l of instruction `it` lands on physical chunk l % CPR of LDS row
-        // row0 + it * DMA_ROW_STEP, so it fetches the logical chunk the swizzle maps there
-        const int row0 = wave * Cfg::ROWS_PER_DMA + lane / CPR;
-        const int last_a = M - 1 - tile_m * BM, last_b = N - 1 - tile_n * BN;  // last valid row of the tile
-#pragma unroll
-        for (int it = 0; it < A_DMA; ++it) {
-            const int row = row0 + it * DMA_ROW_STEP;
-            const int ch = (lane % CPR) ^ pipe_swizzle<Cfg>(row);
-            const int src = (EDGE && row > last_a) ? last_a : row;
-            voff[it] = ((uint32_t)src * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
-        }
-#pragma unroll
-        for (int it = 0; it < B_DMA; ++it) {
-            const int row = row0 + it * DMA_ROW_STEP;
-            const int ch = (lane % CPR) ^ pipe_swizzle<Cfg>(row);
-            const int src = (EDGE && row > last_b) ? last_b : row;
-            voff[A_DMA + it] = ((uint32_t)src * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
-        }
-    }
-    const uint32_t cp_lds = lds_base + wave * 1024;
-    // ---- operand fragment set-up: lane l supplies 8 consecutive k (chunk l / MI of the
-    // step) of row l % MI, for both operands.
-    const int frag_row = lane % MI;
-    const int frag_x = (lane / MI) ^ pipe_swizzle<Cfg>(frag_row);
-    const uint32_t a_frag_off = (wm * Cfg::WM + frag_row) * ROW_BYTES;
-    const uint32_t b_frag_off = B_REGION + (wn * Cfg::WN + frag_row) * ROW_BYTES;
-    // Fragment idx sits idx * MI rows further down.  That never changes bits 0-2 of the
-    // row's bank-line index, and changes bit 3 (which the swizzle folds into bit 0) only
-    // when MI rows are 8 lines: then odd fragments use the chunk index XOR 1.
-    constexpr int ODD_FLIP = ((MI * BK * 2 / 128) % 16 == 8) ? 16 : 0;
-    uint32_t chunk_off[KSTEPS][ODD_FLIP ? 2 : 1];
-#pragma unroll
-    for (int kk = 0; kk < KSTEPS; ++kk) {
-        chunk_off[kk][0] = (uint32_t)((kk * CPS) ^ frag_x) << 4;
-        if (ODD_FLIP) chunk_off[kk][ODD_FLIP ? 1 : 0] = chunk_off[kk][0] ^ ODD_FLIP;
-    }
+    PipeFrame<Cfg, SPLIT, EDGE> frame;
+    if (!frame.init(A, B, M, N, K, k_len, tiles_m, tiles_n, first_block, subdiv, lds_base)) return;
+    const int lane = frame.lane, wave = frame.wave, wm = frame.wm, wn = frame.wn;
+    int tile_m = frame.tile_m, tile_n = frame.tile_n;
+    const int slot = frame.slot, slice = frame.slice, num_k = frame.num_k;
+    const unsigned char *const a_base = frame.a_base, *const b_base = frame.b_base;
+    const uint32_t(&voff)[L] = frame.voff;
+    const uint32_t cp_lds = frame.cp_lds;
 
     // Operand registers.  Every accumulator receives the chunk's KSTEPS MFMAs back to back
     // (a dependent chain: the matrix pipe then keeps the running sum to itself instead of
@@ -228,27 +152,8 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     half8 a_frag[2][KSTEPS][TM];
     half8 b_frag[2][KSTEPS];
     static_assert(TN % 2 == 0, "columns alternate between two B fragment buffers");
-    // Byte address (32-bit LDS offset) of this lane's fragment of A tile 0 / B tile 0 for
-    // step kk, without the ring-buffer base; tile t adds the constant t * MI * ROW_BYTES.
-    uint32_t a_addr[KSTEPS][ODD_FLIP ? 2 : 1], b_addr[KSTEPS][ODD_FLIP ? 2 : 1];
-#pragma unroll
-    for (int kk = 0; kk < KSTEPS; ++kk)
-#pragma unroll
-        for (int f = 0; f < (ODD_FLIP ? 2 : 1); ++f) {
-            a_addr[kk][f] = lds_base + a_frag_off + chunk_off[kk][f];
-            b_addr[kk][f] = lds_base + b_frag_off + chunk_off[kk][f];
-        }
-    static_assert((TN - 1) * MI * ROW_BYTES < 65536 && (TM - 1) * MI * ROW_BYTES < 65536,
-                  "fragment offsets must fit the 16-bit ds_read offset field");
-    auto read_a = [&](auto t_c, uint32_t stage_bytes, auto kk_c) -> half8 {
-        constexpr int t = decltype(t_c)::value, kk = decltype(kk_c)::value;
-        return lds_read16<t * MI * ROW_BYTES>(a_addr[kk][ODD_FLIP ? (t & 1) : 0] + stage_bytes);
-    };
-    auto read_b = [&](auto t_c, uint32_t stage_bytes, auto kk_c) -> half8 {
-        constexpr int t = decltype(t_c)::value, kk = decltype(kk_c)::value;
-        return lds_read16<t * MI * ROW_BYTES>(b_addr[kk][ODD_FLIP ? (t & 1) : 0] + stage_bytes);
-    };
-
+    auto read_a = [&](auto t_c, uint32_t stage_bytes, auto kk_c) -> half8 { return frame.read_a(t_c, stage_bytes, kk_c); };
+    auto read_b = [&](auto t_c, uint32_t stage_bytes, auto kk_c) -> half8 { return frame.read_b(t_c, stage_bytes, kk_c); };
 
     // ---- pipeline.  Chunk c of A lives in A-ring buffer c % SA, of B in B-ring buffer c % SB.
     //
@@ -422,14 +327,14 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             __builtin_amdgcn_sched_barrier(0);
             // operand reads of this block: B fragments of the next column (of the next chunk's
             // column 0 in the last block), then A fragments of the next chunk
-            constexpr int n_b = (Cfg::DBG_MODE != 4 && !(FINAL && last)) ? KSTEPS : 0;
-            constexpr int n_a = (Cfg::DBG_MODE != 4 && !FINAL) ? a_reads_in_block(j) : 0;
+            constexpr int n_b = !(FINAL && last) ? KSTEPS : 0;
+            constexpr int n_a = !FINAL ? a_reads_in_block(j) : 0;
             constexpr int a_first = a_reads_before_block(j);
             static_for<BS>([&](auto sl_c) {
                 constexpr int sl = decltype(sl_c)::value, slot = j * BS + sl;
                 constexpr int i = sl / KSTEPS, kk = sl % KSTEPS;
                 constexpr int rel = slot >= SBAR ? slot - SBAR : slot + NM - SBAR;
-                constexpr int copy = (!FINAL && Cfg::DBG_MODE != 1 && Cfg::DBG_MODE != 4) ? copy_at(rel) : -1;
+                constexpr int copy = !FINAL ? copy_at(rel) : -1;
                 using Tile = std::integral_constant<int, j * TM + i>;
                 if constexpr (copy >= 0) {
                     if constexpr (slot >= SBAR)
@@ -456,17 +361,11 @@ __global__ void __launch_bounds__(Cfg::THREADS)
                 // The sources of the next window, a few scalar instructions at a time in slots that
                 // host nothing else (block 1: no copy of this window's start is issued before the barrier).
                 if constexpr (!FINAL && j == 1 && sl == 3) {
-                    if constexpr (Cfg::DBG_MODE == 2)  // probe build: the same two chunks over and over (L2 hits)
-                        a_off_far = a_off_far == 0 ? BK * 2 : 0;
-                    else
-                        a_off_far = a_off_far + BK * 2 < last_off ? a_off_far + BK * 2 : last_off;
+                    a_off_far = a_off_far + BK * 2 < last_off ? a_off_far + BK * 2 : last_off;
                     a_post = a_base + a_off_far;
                 }
                 if constexpr (!FINAL && j == 1 && sl == 5) {
-                    if constexpr (Cfg::DBG_MODE == 2)
-                        b_off_far = b_off_far == 0 ? BK * 2 : 0;
-                    else
-                        b_off_far = b_off_far + BK * 2 < last_off ? b_off_far + BK * 2 : last_off;
+                    b_off_far = b_off_far + BK * 2 < last_off ? b_off_far + BK * 2 : last_off;
                     b_post = b_base + b_off_far;
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -483,7 +382,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
                 }
                 static_for<KSTEPS>([&](auto kk_c) { lds_landed(b_frag[(j + 1) & 1][decltype(kk_c)::value]); });
             }
-            if constexpr (j == TN - 2 && Cfg::DBG_MODE != 4 && !FINAL) {
+            if constexpr (j == TN - 2 && !FINAL) {
                 static_for<KSTEPS>([&](auto kk_c) {
                     static_for<TM>([&](auto t) { lds_landed(a_frag[NB][decltype(kk_c)::value][decltype(t)::value]); });
                 });
@@ -492,10 +391,6 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         a_pre = a_post;  // what started as this window's start is the next iteration's "rest of the previous window"
         b_pre = b_post;
     };
-    if constexpr (Cfg::TIMESTAMPS) {
-        t_loop = wall_clock64();
-        c_loop = clock64();
-    }
 
     // The loop, unrolled over one period of the two rings and of the A fragment double buffer
     // so that every buffer index is a constant: no index arithmetic or address computation is
@@ -538,10 +433,6 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     int lane_late = lane;
     asm volatile("" : "+v"(lane_late));
     // ---- epilogue: accumulators -> fp16 -> C (through LDS, whole lines per store)
-    if constexpr (Cfg::TIMESTAMPS) {
-        t_epi = wall_clock64();
-        c_epi = clock64();
-    }
     wait_vmcnt<0>();  // the redundant copies of the last iterations: landed before LDS is reused or the wave ends
     if constexpr (SPLIT) {
         __syncthreads();  // every wave has read its last operands: the strips reuse the ring
@@ -559,20 +450,6 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         __syncthreads();
         store_chained_tile<Cfg, EDGE>(lds, C, M, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN, wave, lane_late);
     }
-    if constexpr (Cfg::TIMESTAMPS) {
-      if (probe_out && tid == 0) {
-        __builtin_amdgcn_s_waitcnt(0);
-        long long *t = probe_out + (size_t)blockIdx.x * 8;
-        t[0] = t_begin;
-        t[1] = t_loop;
-        t[2] = t_epi;
-        t[3] = wall_clock64();
-        t[4] = __builtin_amdgcn_s_getreg((31 << 11) | 4);   // HW_ID: wave / simd / cu / sh / se
-        t[5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID
-        t[6] = c_epi - c_loop;
-      }
-    }
-    (void)t_begin, (void)t_loop, (void)t_epi, (void)c_loop, (void)c_epi, (void)probe_out;
 }
 
 }  // namespace hgemm

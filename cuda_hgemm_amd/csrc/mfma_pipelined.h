@@ -21,8 +21,7 @@
 
 namespace hgemm {
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int MI_ = 16, int DBG_ = 0,
-          int EXTRA_A_ = 0>
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int MI_ = 16, int EXTRA_A_ = 0>
 struct PipeConfig : TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true> {
     using Base = TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_DMA, LDS_SWIZZLE, true>;
     // MFMA shape: 32 -> v_mfma_f32_32x32x16_f16, 16 -> v_mfma_f32_16x16x32_f16.  Both move
@@ -34,13 +33,6 @@ struct PipeConfig : TileConfig<BM_, BN_, BK_, WAVES_M_, WAVES_N_, STAGES_, LOAD_
     static constexpr int PKSTEP = MI == 32 ? 16 : 32;               // k covered by one MFMA
     static constexpr int PKSTEPS = BK_ / PKSTEP;
     static constexpr int CPS = PKSTEP / 8;                          // 16-byte chunks per row per step
-    // Timing experiments only (the library instantiates DBG = 0, which compiles none of it):
-    // low three bits: 1 = no copies in the loop, 2 = copies from a fixed K offset, 4 = no operand
-    // reads in the loop; + 16 / + 32 = strip / block tile order regardless of the problem; any
-    // non-zero value also records per-workgroup timestamps into `probe_out`.
-    static constexpr int DBG = DBG_;
-    static constexpr int DBG_MODE = DBG_ & 7;
-    static constexpr bool TIMESTAMPS = DBG_ != 0;
     // Ring depths.  The B ring has STAGES buffers, the A ring STAGES + EXTRA_A: 256x256x64
     // tiles are 32 KB per operand and chunk, so the 160 KB of LDS hold two full stages plus
     // one more A buffer -- the A copies then run two chunks ahead and only the B copies
@@ -269,97 +261,158 @@ __device__ __forceinline__ void store_wave_tile_f32(Get get, unsigned char *lds,
     });
 }
 
+// What both tuned kernels (interleaved below, chained in mfma_chained.h) set up before their loops: which tile
+// and K slice the workgroup computes, the per-lane global offsets of its direct-to-LDS copies, and the LDS
+// addresses its lanes read MFMA operands from.
 // EDGE: M and N need not be multiples of the tile (N % 8 == 0 still, for aligned rows of
 // C).  Copies of rows beyond the matrix are redirected to its last row -- valid memory,
 // products never stored -- which costs nothing inside the loop; only the stores are guarded.
+template <class Cfg, bool SPLIT, bool EDGE>
+struct PipeFrame {
+    static constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
+    static constexpr int KSTEPS = Cfg::PKSTEPS, CPR = Cfg::CPR, CPS = Cfg::CPS, ROW_BYTES = Cfg::ROW_BYTES;
+    static constexpr int A_DMA = Cfg::A_DMA, B_DMA = Cfg::B_DMA, L = A_DMA + B_DMA;
+    static constexpr int B_REGION = Cfg::SA * Cfg::A_BYTES;  // LDS: the A ring (SA buffers), then the B ring (SB buffers)
+    // Fragment idx sits idx * MI rows further down.  That never changes bits 0-2 of the
+    // row's bank-line index, and changes bit 3 (which the swizzle folds into bit 0) only
+    // when MI rows are 8 lines: then odd fragments use the chunk index XOR 1.
+    static constexpr int ODD_FLIP = ((MI * BK * 2 / 128) % 16 == 8) ? 16 : 0;
+    static constexpr int NF = ODD_FLIP ? 2 : 1;
+    static_assert((Cfg::PTN - 1) * MI * ROW_BYTES < 65536 && (Cfg::PTM - 1) * MI * ROW_BYTES < 65536,
+                  "fragment offsets must fit the 16-bit ds_read offset field");
+
+    int lane, wave, wm, wn;
+    int tile_m, tile_n;      // the workgroup's tile (wave-uniform)
+    int slot, slice;         // its position among the launch's tiles and, in a K-sliced launch, its slice
+    int num_k;               // chunks it walks
+    const unsigned char *a_base, *b_base;  // first chunk of the tile's rows of A and of B
+    uint32_t voff[L];        // per-lane byte offset of copy instruction i from a_base (i < A_DMA) or b_base
+    uint32_t cp_lds;         // LDS address the wave's copy instruction 0 fills, without the ring-buffer offset
+    // Byte address (32-bit LDS offset) of this lane's fragment of A tile 0 / B tile 0 for
+    // step kk, without the ring-buffer base; tile t adds the constant t * MI * ROW_BYTES.
+    uint32_t a_addr[KSTEPS][NF], b_addr[KSTEPS][NF];
+
+    // false: this workgroup has no tile (a part of a subdivided tile that lies wholly outside the matrix)
+    __device__ __forceinline__ bool init(const half_t *A, const half_t *B, int M, int N, int K, int k_len, int tiles_m,
+                                         int tiles_n, int first_block, int subdiv, uint32_t lds_base) {
+        const int tid = threadIdx.x;
+        lane = tid & 63;
+        wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
+        const bool blocked = blocked_order(N, K);  // the same in every launch that works on this problem
+        // this workgroup's slot among the launch's positions: slots are dealt so that the workgroups an XCD runs
+        // together are neighbours in the tile order.  A K-sliced launch is one-dimensional as well, slice-major, so
+        // that those neighbours also work on the same slice of K.
+        slice = 0;
+        if constexpr (SPLIT) {
+            const int slices = K / k_len;
+            slice_and_slot_of_workgroup((int)blockIdx.x, (int)gridDim.x / slices, slices, slice, slot);
+            slice = __builtin_amdgcn_readfirstlane(slice);
+        } else {
+            slot = slot_of_workgroup(blocked, (int)blockIdx.x, (int)gridDim.x);
+        }
+        if (subdiv == 0) {
+            // the launch covers positions [first_block, first_block + gridDim.x) of the tile order
+            tile_of_position(blocked, first_block + slot, tiles_m, tiles_n, tile_m, tile_n);
+        } else {
+            // tiles_m x tiles_n is the grid of a larger tile that this one divides sub_m x sub_n times;
+            // consecutive slots take the parts of the tile at position first_block + slot / parts
+            const int sub_m = subdiv >> 8, sub_n = subdiv & 255, parts = sub_m * sub_n;
+            const int part = slot % parts;
+            int parent_m, parent_n;
+            tile_of_position(blocked, first_block + slot / parts, tiles_m, tiles_n, parent_m, parent_n);
+            tile_m = parent_m * sub_m + part / sub_n;
+            tile_n = parent_n * sub_n + part % sub_n;
+            if (tile_m * BM >= M || tile_n * BN >= N) return false;  // the whole workgroup
+        }
+        tile_m = __builtin_amdgcn_readfirstlane(tile_m);  // wave-uniform by construction: keep them in SGPRs
+        tile_n = __builtin_amdgcn_readfirstlane(tile_n);
+        num_k = k_len / BK;
+        const int k_begin = slice * k_len;
+
+        // ---- copies: wave w, instruction i fills LDS rows [(i*WAVES + w)*ROWS_PER_DMA, +ROWS_PER_DMA)
+        a_base = reinterpret_cast<const unsigned char *>(A + (size_t)tile_m * BM * K + k_begin);
+        b_base = reinterpret_cast<const unsigned char *>(B + (size_t)tile_n * BN * K + k_begin);
+        constexpr int DMA_ROW_STEP = Cfg::WAVES * Cfg::ROWS_PER_DMA;
+        {
+            // lane l of instruction `it` lands on physical chunk l % CPR of LDS row
+            // row0 + it * DMA_ROW_STEP, so it fetches the logical chunk the swizzle maps there
+            const int row0 = wave * Cfg::ROWS_PER_DMA + lane / CPR;
+            const int last_a = M - 1 - tile_m * BM, last_b = N - 1 - tile_n * BN;  // last valid row of the tile
+#pragma unroll
+            for (int it = 0; it < A_DMA; ++it) {
+                const int row = row0 + it * DMA_ROW_STEP;
+                const int ch = (lane % CPR) ^ pipe_swizzle<Cfg>(row);
+                const int src = (EDGE && row > last_a) ? last_a : row;
+                voff[it] = ((uint32_t)src * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
+            }
+#pragma unroll
+            for (int it = 0; it < B_DMA; ++it) {
+                const int row = row0 + it * DMA_ROW_STEP;
+                const int ch = (lane % CPR) ^ pipe_swizzle<Cfg>(row);
+                const int src = (EDGE && row > last_b) ? last_b : row;
+                voff[A_DMA + it] = ((uint32_t)src * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
+            }
+        }
+        cp_lds = lds_base + wave * 1024;
+
+        // ---- operand fragments: lane l supplies 8 consecutive k (chunk l / MI of the
+        // step) of row l % MI, for both operands.
+        const int frag_row = lane % MI;
+        const int frag_x = (lane / MI) ^ pipe_swizzle<Cfg>(frag_row);
+        const uint32_t a_frag_off = (wm * Cfg::WM + frag_row) * ROW_BYTES;
+        const uint32_t b_frag_off = B_REGION + (wn * Cfg::WN + frag_row) * ROW_BYTES;
+#pragma unroll
+        for (int kk = 0; kk < KSTEPS; ++kk)
+#pragma unroll
+            for (int f = 0; f < NF; ++f) {
+                const uint32_t chunk_off = ((uint32_t)((kk * CPS) ^ frag_x) << 4) ^ (uint32_t)(f * ODD_FLIP);
+                a_addr[kk][f] = lds_base + a_frag_off + chunk_off;
+                b_addr[kk][f] = lds_base + b_frag_off + chunk_off;
+            }
+        return true;
+    }
+
+    // operand fragment of A / B tile t for MFMA step kk of the chunk in the ring buffer at byte offset stage_bytes
+    template <class TC, class KC>
+    __device__ __forceinline__ half8 read_a(TC, uint32_t stage_bytes, KC) const {
+        constexpr int t = TC::value, kk = KC::value;
+        return lds_read16<t * MI * ROW_BYTES>(a_addr[kk][ODD_FLIP ? (t & 1) : 0] + stage_bytes);
+    }
+    template <class TC, class KC>
+    __device__ __forceinline__ half8 read_b(TC, uint32_t stage_bytes, KC) const {
+        constexpr int t = TC::value, kk = KC::value;
+        return lds_read16<t * MI * ROW_BYTES>(b_addr[kk][ODD_FLIP ? (t & 1) : 0] + stage_bytes);
+    }
+};
+
 template <class Cfg, bool SPLIT = false, bool EDGE = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_pipelined_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
                            float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n,
-                           int first_block, int tail_tiles, int subdiv, long long *probe_out) {
+                           int first_block, int tail_tiles, int subdiv) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
-    constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS, CPR = Cfg::CPR, CPS = Cfg::CPS;
-    constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES, SA = Cfg::SA, SB = Cfg::SB;
+    constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS;
+    constexpr int STAGES = Cfg::STAGES, SA = Cfg::SA, SB = Cfg::SB;
     constexpr int A_BYTES = Cfg::A_BYTES, B_BYTES = Cfg::B_BYTES, B_REGION = SA * A_BYTES;
     constexpr int A_DMA = Cfg::A_DMA, B_DMA = Cfg::B_DMA, L = A_DMA + B_DMA;
     constexpr int NFRAG = TM + TN, NMMA = TM * TN;
     typedef typename MfmaOp<MI>::Acc Acc;
     static_assert(NFRAG <= NMMA, "at most one operand read is issued per MFMA slot");
     static_assert(!SPLIT || MI == 16, "fp32 partial stores are written for the 16x16x32 accumulator layout");
-    long long t_begin = 0, t_loop = 0, t_epi = 0, c_loop = 0, c_epi = 0;
-    if constexpr (Cfg::TIMESTAMPS) t_begin = wall_clock64();
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
-
-    int tile_m, tile_n;
-    // the same in every launch that works on this problem (probe builds can force either order)
-    const bool blocked = (Cfg::DBG & 16) ? false : ((Cfg::DBG & 32) ? true : blocked_order(N, K));
-    // this workgroup's slot among the launch's positions: slots are dealt so that the workgroups an XCD runs
-    // together are neighbours in the tile order.  A K-sliced launch is one-dimensional as well, slice-major, so
-    // that those neighbours also work on the same slice of K.
-    int slot, slice = 0;
-    if constexpr (SPLIT) {
-        const int slices = K / k_len;
-        slice_and_slot_of_workgroup((int)blockIdx.x, (int)gridDim.x / slices, slices, slice, slot);
-        slice = __builtin_amdgcn_readfirstlane(slice);
-    } else {
-        slot = slot_of_workgroup(blocked, (int)blockIdx.x, (int)gridDim.x);
-    }
-    if (subdiv == 0) {
-        // the launch covers positions [first_block, first_block + gridDim.x) of the tile order
-        tile_of_position(blocked, first_block + slot, tiles_m, tiles_n, tile_m, tile_n);
-    } else {
-        // tiles_m x tiles_n is the grid of a larger tile that this one divides sub_m x sub_n times;
-        // consecutive slots take the parts of the tile at position first_block + slot / parts
-        const int sub_m = subdiv >> 8, sub_n = subdiv & 255, parts = sub_m * sub_n;
-        const int part = slot % parts;
-        int parent_m, parent_n;
-        tile_of_position(blocked, first_block + slot / parts, tiles_m, tiles_n, parent_m, parent_n);
-        tile_m = parent_m * sub_m + part / sub_n;
-        tile_n = parent_n * sub_n + part % sub_n;
-        if (tile_m * BM >= M || tile_n * BN >= N) return;  // a part wholly outside the matrix (whole workgroup)
-    }
-    tile_m = __builtin_amdgcn_readfirstlane(tile_m);  // wave-uniform by construction: keep them in SGPRs
-    tile_n = __builtin_amdgcn_readfirstlane(tile_n);
-    const int num_k = k_len / BK;
-    const int k_begin = slice * k_len;
-
-    // ---- copy set-up: wave w, instruction i fills LDS rows [(i*WAVES + w)*ROWS_PER_DMA, +ROWS_PER_DMA)
-    const unsigned char *a_base = reinterpret_cast<const unsigned char *>(A + (size_t)tile_m * BM * K + k_begin);
-    const unsigned char *b_base = reinterpret_cast<const unsigned char *>(B + (size_t)tile_n * BN * K + k_begin);
-    constexpr int DMA_ROW_STEP = Cfg::WAVES * Cfg::ROWS_PER_DMA;
-    uint32_t voff[L];
-    {
-        // lane l of instruction `it` lands on physical chunk l % CPR of LDS row
-        // row0 + it * DMA_ROW_STEP, so it fetches the logical chunk the swizzle maps there
-        const int row0 = wave * Cfg::ROWS_PER_DMA + lane / CPR;
-        const int last_a = M - 1 - tile_m * BM, last_b = N - 1 - tile_n * BN;  // last valid row of the tile
-#pragma unroll
-        for (int it = 0; it < A_DMA; ++it) {
-            const int row = row0 + it * DMA_ROW_STEP;
-            const int ch = (lane % CPR) ^ pipe_swizzle<Cfg>(row);
-            const int src = (EDGE && row > last_a) ? last_a : row;
-            voff[it] = ((uint32_t)src * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
-        }
-#pragma unroll
-        for (int it = 0; it < B_DMA; ++it) {
-            const int row = row0 + it * DMA_ROW_STEP;
-            const int ch = (lane % CPR) ^ pipe_swizzle<Cfg>(row);
-            const int src = (EDGE && row > last_b) ? last_b : row;
-            voff[A_DMA + it] = ((uint32_t)src * (uint32_t)K + (uint32_t)(ch * 8)) * 2u;
-        }
-    }
-    const uint32_t cp_lds = lds_base + wave * 1024;
-    // copy instruction `idx` (0..L-1) of chunk at byte offset kbyte into ring buffer `stage`
-    // LDS is laid out as the A ring (SA buffers) followed by the B ring (SB buffers).
-    // `a_src` / `b_src` already point at the chunk; `dst_a` / `dst_b` are cp_lds plus the
-    // byte offset of the ring buffer to fill.
+    PipeFrame<Cfg, SPLIT, EDGE> frame;
+    if (!frame.init(A, B, M, N, K, k_len, tiles_m, tiles_n, first_block, subdiv, lds_base)) return;
+    const int lane = frame.lane, wave = frame.wave, wm = frame.wm, wn = frame.wn;
+    const int tile_m = frame.tile_m, tile_n = frame.tile_n, slot = frame.slot, slice = frame.slice;
+    const int num_k = frame.num_k;
+    const unsigned char *const a_base = frame.a_base, *const b_base = frame.b_base;
+    const uint32_t(&voff)[L] = frame.voff;
+    const uint32_t cp_lds = frame.cp_lds;
+    // copy instruction `idx` (0..L-1) of a chunk: `a_src` / `b_src` already point at the chunk; `dst_a` / `dst_b`
+    // are cp_lds plus the byte offset of the ring buffer to fill.
     auto dma_one = [&](auto idx_c, const unsigned char *a_src, const unsigned char *b_src, uint32_t dst_a,
                        uint32_t dst_b) {
         constexpr int idx = decltype(idx_c)::value;
@@ -368,23 +421,6 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         else
             dma_load16_sv<(idx - A_DMA) * Cfg::WAVES * 1024>(b_src, voff[idx], dst_b);
     };
-
-    // ---- operand fragment set-up: lane l supplies 8 consecutive k (chunk l / MI of the
-    // step) of row l % MI, for both operands.
-    const int frag_row = lane % MI;
-    const int frag_x = (lane / MI) ^ pipe_swizzle<Cfg>(frag_row);
-    const uint32_t a_frag_off = (wm * Cfg::WM + frag_row) * ROW_BYTES;
-    const uint32_t b_frag_off = B_REGION + (wn * Cfg::WN + frag_row) * ROW_BYTES;
-    // Fragment idx sits idx * MI rows further down.  That never changes bits 0-2 of the
-    // row's bank-line index, and changes bit 3 (which the swizzle folds into bit 0) only
-    // when MI rows are 8 lines: then odd fragments use the chunk index XOR 1.
-    constexpr int ODD_FLIP = ((MI * BK * 2 / 128) % 16 == 8) ? 16 : 0;
-    uint32_t chunk_off[KSTEPS][ODD_FLIP ? 2 : 1];
-#pragma unroll
-    for (int kk = 0; kk < KSTEPS; ++kk) {
-        chunk_off[kk][0] = (uint32_t)((kk * CPS) ^ frag_x) << 4;
-        if (ODD_FLIP) chunk_off[kk][ODD_FLIP ? 1 : 0] = chunk_off[kk][0] ^ ODD_FLIP;
-    }
 
     // Operand registers.  MFMAs run B-major (all A tiles against B tile 0, then B tile 1,
     // ...): a B fragment is dead after TM MFMAs and is reloaded in place for the next step
@@ -396,26 +432,8 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     constexpr int NSB = TN - NDB;          // leading B tiles reloaded in place
     half8 b_frag[NSB > 0 ? NSB : 1];
     half8 b_last[2][NDB];
-    // Byte address (32-bit LDS offset) of this lane's fragment of A tile 0 / B tile 0 for
-    // step kk, without the ring-buffer base; tile t adds the constant t * MI * ROW_BYTES.
-    uint32_t a_addr[KSTEPS][ODD_FLIP ? 2 : 1], b_addr[KSTEPS][ODD_FLIP ? 2 : 1];
-#pragma unroll
-    for (int kk = 0; kk < KSTEPS; ++kk)
-#pragma unroll
-        for (int f = 0; f < (ODD_FLIP ? 2 : 1); ++f) {
-            a_addr[kk][f] = lds_base + a_frag_off + chunk_off[kk][f];
-            b_addr[kk][f] = lds_base + b_frag_off + chunk_off[kk][f];
-        }
-    static_assert((TN - 1) * MI * ROW_BYTES < 65536 && (TM - 1) * MI * ROW_BYTES < 65536,
-                  "fragment offsets must fit the 16-bit ds_read offset field");
-    auto read_a = [&](auto t_c, uint32_t stage_bytes, auto kk_c) -> half8 {
-        constexpr int t = decltype(t_c)::value, kk = decltype(kk_c)::value;
-        return lds_read16<t * MI * ROW_BYTES>(a_addr[kk][ODD_FLIP ? (t & 1) : 0] + stage_bytes);
-    };
-    auto read_b = [&](auto t_c, uint32_t stage_bytes, auto kk_c) -> half8 {
-        constexpr int t = decltype(t_c)::value, kk = decltype(kk_c)::value;
-        return lds_read16<t * MI * ROW_BYTES>(b_addr[kk][ODD_FLIP ? (t & 1) : 0] + stage_bytes);
-    };
+    auto read_a = [&](auto t_c, uint32_t stage_bytes, auto kk_c) -> half8 { return frame.read_a(t_c, stage_bytes, kk_c); };
+    auto read_b = [&](auto t_c, uint32_t stage_bytes, auto kk_c) -> half8 { return frame.read_b(t_c, stage_bytes, kk_c); };
     // every outstanding operand read has landed; ties all fragments of buffer `buf`
     auto wait_operands = [&](auto buf_c) {
         constexpr int buf = decltype(buf_c)::value;
@@ -518,17 +536,13 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     // NEXT: chunk kt+1 exists (the barrier is needed and its operands are prefetched).
     // cur_a / cur_b (ring buffers holding chunk kt) are plain ints or, in the unrolled steady
     // state, compile-time constants: then every LDS address below is a constant offset.
-    auto iteration = [&](int kt, auto cur_a_arg, auto cur_b_arg, auto issue_tag, auto next_tag) {
+    auto iteration = [&](auto cur_a_arg, auto cur_b_arg, auto issue_tag, auto next_tag) {
         constexpr bool ISSUE = decltype(issue_tag)::value, NEXT = decltype(next_tag)::value;
         const int cur_a = ring_index(cur_a_arg), cur_b = ring_index(cur_b_arg);
         const int nxt_a = (cur_a + 1 == SA) ? 0 : cur_a + 1;
         const int nxt_b = (cur_b + 1 == SB) ? 0 : cur_b + 1;
         const int fill_a = (cur_a + FILL_OFF_A) % SA, fill_b = (cur_b + FILL_OFF_B) % SB;
         const unsigned char *a_src = a_next, *b_src = b_next;  // chunk kt + AHEAD
-        if constexpr (Cfg::DBG_MODE == 2) {
-            a_src = a_base + (kt & 1) * BK * 2;
-            b_src = b_base + (kt & 1) * BK * 2;
-        }
         if constexpr (ISSUE) {
             a_next += BK * 2;
             b_next += BK * 2;
@@ -554,13 +568,13 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             using SrcKK = std::integral_constant<int, (last ? 0 : kk + 1)>;
             static_for<NMMA>([&](auto idx_c) {
                 constexpr int idx = decltype(idx_c)::value;
-                constexpr int copy = (ISSUE && Cfg::DBG_MODE != 1 && Cfg::DBG_MODE != 4) ? copy_in_slot(kk * NMMA + idx) : -1;
+                constexpr int copy = ISSUE ? copy_in_slot(kk * NMMA + idx) : -1;
                 if constexpr (copy >= 0)
                     mma_and_copy(idx_c, std::integral_constant<int, fb>{}, std::integral_constant<int, copy>{}, a_src,
                                  b_src, dst_a, dst_b);
                 else
                     mma_one(idx_c, std::integral_constant<int, fb>{});
-                if constexpr (prefetch && Cfg::DBG_MODE != 4) {
+                if constexpr (prefetch) {
                     // One operand read per slot at most, spread out (an LDS read in the slot
                     // right after another one stalls MFMA issue): A tile t for the next step
                     // at slot RS*t + 2, the double-buffered trailing B tiles at slots 0 and
@@ -580,13 +594,9 @@ __global__ void __launch_bounds__(Cfg::THREADS)
             // Every operand read issued during this step has landed before control leaves
             // it.  The wait sits here, not at the top of the next step, so that no register
             // copy the compiler may place on a loop edge can see a fragment in flight.
-            if constexpr (prefetch && Cfg::DBG_MODE != 4) wait_operands(std::integral_constant<int, nb>{});
+            if constexpr (prefetch) wait_operands(std::integral_constant<int, nb>{});
         });
     };
-    if constexpr (Cfg::TIMESTAMPS) {
-        t_loop = wall_clock64();
-        c_loop = clock64();
-    }
     using T = std::true_type;
     using F = std::false_type;
 
@@ -597,7 +607,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     for (; kt + PERIOD <= num_k - AHEAD; kt += PERIOD)
         static_for<PERIOD>([&](auto u_c) {
             constexpr int u = decltype(u_c)::value;
-            iteration(kt + u, std::integral_constant<int, u % SA>{}, std::integral_constant<int, u % SB>{}, T{}, T{});
+            iteration(std::integral_constant<int, u % SA>{}, std::integral_constant<int, u % SB>{}, T{}, T{});
         });
     int cur_a = 0, cur_b = 0;  // kt is a multiple of the period here
     auto advance = [&] {
@@ -605,14 +615,14 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         cur_b = (cur_b + 1 == SB) ? 0 : cur_b + 1;
     };
     for (; kt < num_k - AHEAD; ++kt) {  // chunk kt+AHEAD exists
-        iteration(kt, cur_a, cur_b, T{}, T{});
+        iteration(cur_a, cur_b, T{}, T{});
         advance();
     }
     for (; kt < num_k - 1; ++kt) {  // drain: nothing left to copy
-        iteration(kt, cur_a, cur_b, F{}, T{});
+        iteration(cur_a, cur_b, F{}, T{});
         advance();
     }
-    iteration(kt, cur_a, cur_b, F{}, F{});
+    iteration(cur_a, cur_b, F{}, F{});
 
     // The MFMAs were issued from assembly, so the compiler neither knows their latency nor
     // sees any reason to keep its own accumulator reads behind them.  Let the last results
@@ -623,10 +633,6 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         static_for<TN>([&](auto j_c) { pin_accumulator(acc[decltype(i_c)::value][decltype(j_c)::value]); });
     });
     // ---- epilogue: accumulators -> fp16 -> C (through LDS, whole lines per store)
-    if constexpr (Cfg::TIMESTAMPS) {
-        t_epi = wall_clock64();
-        c_epi = clock64();
-    }
     if constexpr (SPLIT) {
         __syncthreads();  // every wave has read its last operands: the strips reuse the ring
         auto get = [&](auto i_c, auto j_c) -> floatx4 { return acc[decltype(i_c)::value][decltype(j_c)::value]; };
@@ -644,20 +650,6 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         store_wave_tile<Cfg, Acc, EDGE>(acc, lds, C, M, N, tile_m * BM + wm * Cfg::WM, tile_n * BN + wn * Cfg::WN,
                                         wave, lane);
     }
-    if constexpr (Cfg::TIMESTAMPS) {
-      if (probe_out && tid == 0) {
-        __builtin_amdgcn_s_waitcnt(0);
-        long long *t = probe_out + (size_t)blockIdx.x * 8;
-        t[0] = t_begin;
-        t[1] = t_loop;
-        t[2] = t_epi;
-        t[3] = wall_clock64();
-        t[4] = __builtin_amdgcn_s_getreg((31 << 11) | 4);   // HW_ID: wave / simd / cu / sh / se
-        t[5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID
-        t[6] = c_epi - c_loop;
-      }
-    }
-    (void)t_begin, (void)t_loop, (void)t_epi, (void)c_loop, (void)c_epi, (void)probe_out;
 }
 
 // Shapes a pipelined kernel accepts with guarded edges: any M, N a multiple of 8 (rows of C
@@ -731,7 +723,7 @@ bool use_chained(PipeKernel which, size_t workgroups, size_t k_len) {
 // as in the kernel.
 template <class Cfg, bool SPLIT, bool EDGE>
 void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial, size_t M, size_t N, size_t K,
-                           int splits, long long *probe_out, int first_block = 0, int blocks = -1, int tail_tiles = 0,
+                           int splits, int first_block = 0, int blocks = -1, int tail_tiles = 0,
                            PipeKernel which = PipeKernel::Auto) {
     constexpr int subdiv = 0;
     static bool configured = [] {
@@ -754,7 +746,7 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
             hgemm_chained_kernel<Cfg, SPLIT, EDGE><<<dim3(blocks * splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
                 reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
                 partial, (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, first_block, tail_tiles,
-                subdiv, probe_out);
+                subdiv);
             HGEMM_CHECK_HIP_ERROR(hipGetLastError());
             return;
         }
@@ -762,7 +754,7 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
     HGEMM_CHECK_MSG(which != PipeKernel::Chained, "this tile has no chained kernel");
     hgemm_pipelined_kernel<Cfg, SPLIT, EDGE><<<dim3(blocks * splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), partial,
-        (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, first_block, tail_tiles, subdiv, probe_out);
+        (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, first_block, tail_tiles, subdiv);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 
@@ -781,12 +773,12 @@ void launch_pipelined_with_tail(const void *A, const void *B, void *C, float *pa
                     "%s (tail in %d K slices) needs N %% 8 == 0, slice %% %d == 0, slice >= %d (got M=%zu N=%zu K=%zu)",
                     name, tail_splits, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
     if (Cfg::supports(M, N, K)) {
-        launch_pipelined_impl<Cfg, false, false>(A, B, C, nullptr, M, N, K, 1, nullptr, 0, head);
-        launch_pipelined_impl<Cfg, true, false>(A, B, nullptr, partial, M, N, K, tail_splits, nullptr, head, tail_tiles,
+        launch_pipelined_impl<Cfg, false, false>(A, B, C, nullptr, M, N, K, 1, 0, head);
+        launch_pipelined_impl<Cfg, true, false>(A, B, nullptr, partial, M, N, K, tail_splits, head, tail_tiles,
                                                 tail_tiles);
     } else {
-        launch_pipelined_impl<Cfg, false, true>(A, B, C, nullptr, M, N, K, 1, nullptr, 0, head);
-        launch_pipelined_impl<Cfg, true, true>(A, B, nullptr, partial, M, N, K, tail_splits, nullptr, head, tail_tiles,
+        launch_pipelined_impl<Cfg, false, true>(A, B, C, nullptr, M, N, K, 1, 0, head);
+        launch_pipelined_impl<Cfg, true, true>(A, B, nullptr, partial, M, N, K, tail_splits, head, tail_tiles,
                                                tail_tiles);
     }
     constexpr int PIECES = Cfg::BM * Cfg::BN / 8;
@@ -797,16 +789,16 @@ void launch_pipelined_with_tail(const void *A, const void *B, void *C, float *pa
 
 template <class Cfg>
 void launch_pipelined(const void *A, const void *B, void *C, size_t M, size_t N, size_t K, const char *name,
-                      long long *probe_out = nullptr, PipeKernel which = PipeKernel::Auto) {
+                      PipeKernel which = PipeKernel::Auto) {
     check_operands(A, B, C, M, N, K);
     if (Cfg::supports(M, N, K)) {
-        launch_pipelined_impl<Cfg, false, false>(A, B, C, nullptr, M, N, K, 1, probe_out, 0, -1, 0, which);
+        launch_pipelined_impl<Cfg, false, false>(A, B, C, nullptr, M, N, K, 1, 0, -1, 0, which);
         return;
     }
     HGEMM_CHECK_MSG(pipelined_supports_edges<Cfg>(M, N, K),
                     "%s needs N %% 8 == 0, K %% %d == 0, K >= %d (got M=%zu N=%zu K=%zu)", name, Cfg::BK,
                     Cfg::BK * Cfg::STAGES, M, N, K);
-    launch_pipelined_impl<Cfg, false, true>(A, B, C, nullptr, M, N, K, 1, probe_out, 0, -1, 0, which);
+    launch_pipelined_impl<Cfg, false, true>(A, B, C, nullptr, M, N, K, 1, 0, -1, 0, which);
 }
 
 // K split into `splits` slices: fp32 partial sums of slice s go to partial[s][M][N] (the
@@ -817,13 +809,13 @@ void launch_pipelined_split(const void *A, const void *B, float *partial, size_t
     HGEMM_CHECK(splits >= 1 && K % (size_t)splits == 0 && partial != nullptr);
     const size_t k_len = K / (size_t)splits;
     if (Cfg::supports(M, N, k_len)) {
-        launch_pipelined_impl<Cfg, true, false>(A, B, nullptr, partial, M, N, K, splits, nullptr);
+        launch_pipelined_impl<Cfg, true, false>(A, B, nullptr, partial, M, N, K, splits);
         return;
     }
     HGEMM_CHECK_MSG(pipelined_supports_edges<Cfg>(M, N, k_len),
                     "%s (K in %d slices) needs N %% 8 == 0, slice %% %d == 0, slice >= %d (got M=%zu N=%zu K=%zu)",
                     name, splits, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
-    launch_pipelined_impl<Cfg, true, true>(A, B, nullptr, partial, M, N, K, splits, nullptr);
+    launch_pipelined_impl<Cfg, true, true>(A, B, nullptr, partial, M, N, K, splits);
 }
 
 // Whole rounds of workgroups on the Parent tile, the last `tail_tiles` workgroup ids of its
@@ -844,9 +836,9 @@ void launch_pipelined_with_subtiles(const void *A, const void *B, void *C, size_
                     "%s needs N %% 8 == 0, K %% 64 == 0, K >= %d (got M=%zu N=%zu K=%zu)", name,
                     64 * (Parent::STAGES > Child::STAGES ? Parent::STAGES : Child::STAGES), M, N, K);
     if (Parent::supports(M, N, K))
-        launch_pipelined_impl<Parent, false, false>(A, B, C, nullptr, M, N, K, 1, nullptr, 0, head);
+        launch_pipelined_impl<Parent, false, false>(A, B, C, nullptr, M, N, K, 1, 0, head);
     else
-        launch_pipelined_impl<Parent, false, true>(A, B, C, nullptr, M, N, K, 1, nullptr, 0, head);
+        launch_pipelined_impl<Parent, false, true>(A, B, C, nullptr, M, N, K, 1, 0, head);
     const bool edge = !Child::supports(M, N, K);
     auto kernel = edge ? &hgemm_pipelined_kernel<Child, false, true> : &hgemm_pipelined_kernel<Child, false, false>;
     static bool configured = [] {
@@ -859,7 +851,7 @@ void launch_pipelined_with_subtiles(const void *A, const void *B, void *C, size_
     (void)configured;
     kernel<<<dim3(tail_tiles * sub_m * sub_n), dim3(Child::THREADS), Child::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), nullptr,
-        (int)M, (int)N, (int)K, (int)K, tiles_m, tiles_n, head, 0, (sub_m << 8) | sub_n, nullptr);
+        (int)M, (int)N, (int)K, (int)K, tiles_m, tiles_n, head, 0, (sub_m << 8) | sub_n);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 

@@ -142,11 +142,17 @@ const char *hgemm_kernel_name(int kernel);
  * and live until hgemm_release_workspace or the end of the process (the reference keeps its
  * vendor handle the same way, src/cublas_tensor_op.cu:18).  Each is allocated ONCE, at its
  * cap (512 MiB of partial sums, 1 GiB of operand copies), by the first call that needs it:
- * that one call contains a hipMalloc; no later call allocates, frees or synchronises.
- * Callers that cannot have even that (a timed loop, a stream being captured) reserve
- * beforehand.  If the memory cannot be had, hgemm_auto runs the best plan that needs none.
- * Entry points may be called from several host threads; the workspaces are shared, so
- * calls that overlap on one device must be ordered on its null stream, as they are. */
+ * that one call contains a hipMalloc; no later call frees or synchronises, and none
+ * allocates unless that first hipMalloc was refused (then the size the plan needs is tried
+ * once; refused sizes are remembered and not asked for again).  Callers that cannot have
+ * even that (a timed loop) reserve beforehand.  If the memory cannot be had, hgemm_auto
+ * runs the best plan that needs none.
+ * Entry points may be called from several host threads.  The workspaces are shared: the
+ * library enqueues the launches of a plan that uses one under a lock, and since every
+ * launch goes to the null stream, which runs launches in the order they were enqueued, one
+ * call's partial sums are consumed before the next call's overwrite them.
+ * hgemm_reserve_workspace and hgemm_release_workspace wait for the device before they free
+ * anything and take the same lock. */
 /* Allocates the current device's workspaces now: each at least as large as asked, and at
  * least its cap, unless 0 is asked (that buffer is then left alone).  Returns 0, or 1 if
  * device memory ran out. */
@@ -157,16 +163,22 @@ void hgemm_release_workspace(void);
  * that hgemm_auto's plan for the shape uses. */
 size_t hgemm_auto_workspace_bytes(size_t M, size_t N, size_t K, size_t *operand_bytes);
 
-/* hgemm_auto for callers that cannot allocate device memory (code under HIP graph capture,
- * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Runs
+/* hgemm_auto for callers that cannot allocate device memory (serving loops, harnesses that
+ * forbid hipMalloc).  No counterpart in the reference.  Like every entry point it launches
+ * on the null stream, which cannot be captured into a HIP graph; what it guarantees is that
+ * no call performs a hipMalloc or hipFree (its first call on a device looks up the array's
+ * address and sets kernel attributes, which allocate nothing).  Runs
  * the same plan as hgemm_auto, hence the same result bit for bit, but keeps partial sums and
  * padded operand copies in a fixed array of HGEMM_STATIC_WORKSPACE_BYTES inside the library's
  * code object (every GPU the library runs on holds one copy until the process ends) and
  * calls no hipMalloc, hipFree or other allocating routine.  Returns 0, or 1 -- with a
  * message on stderr and nothing launched -- when the plan needs more than the array holds
  * (hgemm_auto_workspace_bytes tells beforehand).  Other contract violations end the process
- * as everywhere.  All calls on one GPU share that GPU's array: calls that overlap on a GPU
- * (different streams or host threads) race; calls on the null stream are ordered. */
+ * as everywhere.  All calls on one GPU share that GPU's array, which keeps the last call's
+ * contents (nothing in it has to start at zero: every kernel reads only what an earlier
+ * kernel of the same call wrote in full).  Calls from several host threads are enqueued one
+ * plan at a time and the null stream orders them; work a caller moves to other streams so
+ * that two calls overlap on one GPU would race on the array. */
 #define HGEMM_STATIC_WORKSPACE_BYTES ((size_t)64 << 20)
 int hgemm_auto_static_workspace(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N,
                                 size_t K);
