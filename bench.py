@@ -6,11 +6,16 @@ A step is one call of ``hgemm_auto`` (C = A.B^T, fp16 in/out, fp32 accumulate) o
 headline configuration M = N = K = 8192 with uniform[-1,1) inputs already resident in HBM.
 Before anything is timed the device is brought to its steady power state with 300 ms of
 vendor GEMM launches (``--settle-ms``); then come ``--warmup`` untimed and ``--steps`` timed
-calls, bracketed by HIP events on the stream the kernels run on.
+calls, bracketed by HIP events on the stream the kernels run on, and by two samples of the
+shader-cycle counter, which give the clock the part actually sustained during those steps.
 Prints one JSON line: TFLOPS = 2*M*N*K / t (reference src/common/tester.h:96-97), the
-roofline fraction against the dense FP16 MFMA peak, hipBLASLt timed beside it as the vendor
-line (never part of the measured path), and the CPU checker timed on a bounded slab of the
-same product on this box's host cores.
+roofline fraction against the dense FP16 MFMA peak, the same work per shader cycle and CU
+(the figure that does not depend on how far a particular board lowers its clock under its
+power limit), hipBLASLt timed beside it as the vendor line (never part of the measured path),
+and the CPU checker timed on a bounded slab of the same product on this box's host cores.
+
+The process imports no PyTorch: device memory comes from ``cuda_hgemm_amd.hipmem``, so every
+ROCm library in it, the vendor's hipBLASLt included, is the system's.
 
 ``--sweep`` additionally runs every configuration of the specification (squares
 256...16384, the two FFN rectangles, the decode shapes with rotating operands), prints the
@@ -22,80 +27,78 @@ import os
 import sys
 import time
 
+import numpy as np
+
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = 2500.0   # MI355X dense FP16 MFMA, published
 PEAK_GBPS = 8000.0     # MI355X HBM3E, published
+# v_mfma_f32_16x16x32_f16: 16*16*32*2 flop in 16 cycles on each of a CU's 4 SIMDs
+PEAK_FLOP_PER_CYCLE_PER_CU = 4 * (16 * 16 * 32 * 2) / 16
+NOMINAL_GHZ = 2.4
+SUSTAINED_STEPS = 100  # a run shorter than this also reports a leg of this length
 M = N = K = 8192
 
 
-def _inputs(torch, dev, m, n, k, seed, dist_a="uniform", dist_b="uniform"):
-    g = torch.Generator(device=dev).manual_seed(seed)
-
-    def draw(rows, cols, dist):
-        if dist == "uniform":
-            return (torch.rand((rows, cols), device=dev, generator=g, dtype=torch.float32) * 2.0 - 1.0).half()
-        sigma = {"normal": 1.0, "weights": 0.02}[dist]
-        return (torch.randn((rows, cols), device=dev, generator=g, dtype=torch.float32) * sigma).half()
-
-    return draw(m, k, dist_a), draw(n, k, dist_b)
+def _uniform_fp16(rng, rows, cols):
+    """uniform[-1, 1) rounded to fp16, as the reference fills its matrices (src/common/matrix.h:30-33)."""
+    out = np.empty((rows, cols), np.float16)
+    step = max(1, (1 << 24) // cols)
+    for r in range(0, rows, step):  # in slabs: no full-size fp32 temporary
+        out[r:r + step] = rng.random((min(step, rows - r), cols), dtype=np.float32) * 2.0 - 1.0
+    return out
 
 
-def _time_ms(torch, lib, fn, As, Bs, Cs, m, n, k, warmup, steps):
-    """Events on the null stream around `steps` back-to-back launches (Tester::profile)."""
+def _time_ms(lib, hipmem, fn, As, Bs, Cs, m, n, k, warmup, steps, clock=False):
+    """Events on the null stream around `steps` back-to-back launches (Tester::profile);
+    `clock`: also the shader clock sustained over exactly those launches."""
     if warmup:
         lib.profile_fn_rotating_ms(fn, As, Bs, Cs, m, n, k, 0, warmup)
-    torch.cuda.synchronize()
+    hipmem.synchronize()
     t0 = time.perf_counter()
+    if clock:
+        lib.clock_mark(0)
     ms = lib.profile_fn_rotating_ms(fn, As, Bs, Cs, m, n, k, 0, steps)
-    torch.cuda.synchronize()
+    if clock:
+        lib.clock_mark(1)
+    hipmem.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return ms, wall_ms
+    return ms, wall_ms, (lib.clock_between_marks() if clock else None)
 
 
-def _cpu_baseline(torch, A, B, C, budget_s=12.0):
+def _cpu_baseline(A_host, B_host, C_host, budget_s=12.0):
     """The CPU checker (fp32-accumulate blocked GEMM, all host cores) on a slab of complete
     output rows of the same product; also checks those rows of the GPU result."""
-    import numpy as np
     from oracle import oracle
-    k = A.shape[1]
-    n = B.shape[0]
-    Bf = oracle.f16_to_f32(B.view(torch.int16).cpu().numpy().view(np.uint16))
+    k = A_host.shape[1]
+    n = B_host.shape[0]
+    Bf = oracle.f16_to_f32(B_host)
     rows = 128
-    A_host = A.view(torch.int16).cpu().numpy().view(np.uint16)
     secs, _ = oracle.time_sgemm_nt(oracle.f16_to_f32(A_host[:rows]), Bf)          # rate probe
     rate = 2.0 * rows * n * k / secs
-    rows = int(min(A.shape[0], max(rows, (budget_s * rate / (2.0 * n * k)) // 64 * 64)))
+    rows = int(min(A_host.shape[0], max(rows, (budget_s * rate / (2.0 * n * k)) // 64 * 64)))
     Af = oracle.f16_to_f32(A_host[:rows])
     secs, Cf = oracle.time_sgemm_nt(Af, Bf)
     ref = oracle.f32_to_f16(Cf)
-    got = C[:rows].view(torch.int16).cpu().numpy().view(np.uint16)
-    chk = oracle.check(got, ref, k)
+    chk = oracle.check(np.ascontiguousarray(C_host[:rows]), ref, k)
     flops = 2.0 * rows * n * k
     return {"value": flops / secs * 1e-12, "unit": "TFLOPS", "cores": oracle.num_threads(), "kind": "port",
-            "sample": f"rows [0,{rows}) of the {A.shape[0]}x{n}x{k} product, full N and K "
+            "what": "the CPU checker's blocked fp32-accumulate GEMM (the reference has no host GEMM of its own)",
+            "sample": f"rows [0,{rows}) of the {A_host.shape[0]}x{n}x{k} product, full N and K "
                       f"({flops:.3e} flop in {secs:.2f} s, operands pre-converted to fp32)",
             "seconds": secs}, chk
 
 
-def _loaded_library(needle: str):
-    """Path of the shared object whose file name starts with `needle`, as mapped into this process.  PyTorch wheels carry
-    their own libhipblaslt.so.1; imported first, that copy answers the comparator's dependency on the same soname, so
-    the comparator of this process is not necessarily the system ROCm's (the C++ driver links that one)."""
-    try:
-        with open("/proc/self/maps") as f:
-            paths = {line.split()[-1] for line in f if "/" in line and line.rsplit("/", 1)[-1].lower().startswith(needle)}
-        return sorted(paths)[0] if paths else None
-    except OSError:
-        return None
+TRAFFIC_PROFILE = os.path.join("profiles", "hgemm_chained_256x256x64_square8192_hbm_traffic.txt")
 
 
 def _traffic_bytes():
-    """Bytes per launch of the dominant kernel between L2 and the memory fabric, from the
-    committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary under profiles/ (None if absent)."""
-    path = os.path.join(ROOT, "profiles", "hgemm_chained_256x256x64_square8192_hbm_traffic.txt")
+    """Bytes per launch of the dominant kernel between L2 and the memory fabric.  Hardware
+    counters cannot be read from inside the timed process, so this is the figure of the
+    committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary (None if absent), labelled as such."""
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
     try:
         with open(path) as f:
             for line in f:
@@ -122,22 +125,25 @@ def main():
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (a GEMM shards over N or M with no "
                  "exchange; run one process per GPU on its own share). Use --gpus 1.")
 
-    import torch
     import cuda_hgemm_amd
-    lib = cuda_hgemm_amd.library()          # raises if the HIP library is missing: no fallback
-    vendor = cuda_hgemm_amd.vendor_library()
-    dev = torch.device("cuda:0")
-    props = torch.cuda.get_device_properties(0)
+    from cuda_hgemm_amd import hipmem
+    lib = cuda_hgemm_amd.library(torch_runtime=False)     # raises if the HIP library is missing: no fallback
+    vendor = cuda_hgemm_amd.vendor_library(torch_runtime=False)
+    if hipmem.device_count() < 1:
+        sys.exit("bench.py needs a GPU: none is visible")
 
-    A, B = _inputs(torch, dev, M, N, K, 20230212)
-    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
+    rng = np.random.default_rng(20230212)
+    A_host, B_host = _uniform_fp16(rng, M, K), _uniform_fp16(rng, N, K)
+    A, B = hipmem.DeviceArray.from_host(A_host), hipmem.DeviceArray.from_host(B_host)
+    C = hipmem.DeviceArray((M, N)).fill_bytes(0xFF)       # fp16 NaN: an element left unwritten fails the check
+    Cv = hipmem.DeviceArray((M, N))
     auto = lib.variant_fn("hgemm_auto")
-    Cv = torch.empty_like(C)
 
     # One call of each entry point before anything else: the first call of a kernel loads its
     # code object, which takes the host milliseconds during which the device falls idle -- and a
     # power-managed part answers the next burst of matrix work with a clock excursion that lasts
-    # some thirty launches (seen in the kernel trace as 0.70 -> 0.98 -> 0.70 ms per launch).
+    # some thirty launches (seen in the kernel trace as 0.70 -> 0.98 -> 0.70 ms per launch).  The
+    # vendor's first call is also where it times its candidate kernels and keeps the fastest.
     lib.profile_fn_rotating_ms(auto, [A], [B], [C], M, N, K, 0, 1)
     lib.profile_fn_rotating_ms(vendor.fn(), [A], [B], [Cv], M, N, K, 0, 1)
     # From idle the part needs some tens of milliseconds of matrix work to settle on its steady
@@ -151,17 +157,28 @@ def main():
     # Order of the reference's driver: the vendor GEMM is evaluated first (src/main.cu:100), the
     # kernels under test after it.  The part is power-managed and settles only after some tens
     # of launches, so both are timed twice, alternating, and every pass is reported.
-    vms, _ = _time_ms(torch, lib, vendor.fn(), [A], [B], [Cv], M, N, K, args.warmup, args.steps)
-    ms, wall_ms = _time_ms(torch, lib, auto, [A], [B], [C], M, N, K, args.warmup, args.steps)
+    vms, _, vclk = _time_ms(lib, hipmem, vendor.fn(), [A], [B], [Cv], M, N, K, args.warmup, args.steps, clock=True)
+    ms, wall_ms, clk = _time_ms(lib, hipmem, auto, [A], [B], [C], M, N, K, args.warmup, args.steps, clock=True)
     tflops = lib.tflops(M, N, K, ms)
-    out = C.clone()
-    vms2, _ = _time_ms(torch, lib, vendor.fn(), [A], [B], [Cv], M, N, K, args.warmup, args.steps)
-    ms2, _ = _time_ms(torch, lib, auto, [A], [B], [C], M, N, K, args.warmup, args.steps)
-    deterministic = bool(torch.equal(out, C))
+    out = C.to_host()
+    vms2, _, _ = _time_ms(lib, hipmem, vendor.fn(), [A], [B], [Cv], M, N, K, args.warmup, args.steps)
+    ms2, _, _ = _time_ms(lib, hipmem, auto, [A], [B], [C], M, N, K, args.warmup, args.steps)
+    deterministic = bool(np.array_equal(out, C.to_host()))
     vendor_tflops = lib.tflops(M, N, K, min(vms, vms2))   # the better of its passes is the 100 % line
+    # `value` is the leg the driver asked for (--steps); a run shorter than 100 steps still sits
+    # on the part's thermal ramp, so the sustained figure is measured and reported beside it.
+    if args.steps >= SUSTAINED_STEPS:
+        sustained_ms, sustained_clk = ms, clk
+    else:
+        sustained_ms, _, sustained_clk = _time_ms(lib, hipmem, auto, [A], [B], [C], M, N, K, 0, SUSTAINED_STEPS,
+                                                  clock=True)
 
     plan = lib.auto_plan(M, N, K)
     flops = 2.0 * M * N * K
+    cus = hipmem.compute_units()
+    ghz = clk["mhz"] * 1e-3
+    flop_per_cycle_per_cu = flops / (ms * 1e-3) / (ghz * 1e9) / cus
+    traffic = _traffic_bytes()
     result = {
         "metric": "TFLOPS at M=N=K=8192 (square HGEMM, fp16 in/out, fp32 accumulate)",
         "value": tflops, "unit": "TFLOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -170,23 +187,40 @@ def main():
         "config": {"workload": "square HGEMM M=N=K=8192, A row-major, B column-major (N rows of K), C row-major",
                    "entry_point": "hgemm_auto", "kernel": plan["kernel"] + (", chained accumulation" if plan["chained"] else ""),
                    "k_slices": plan["splits"],
-                   "device": props.name, "compute_units": props.multi_processor_count},
+                   "device": hipmem.device_name(), "compute_units": cus},
         "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) * 1e-12, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flops / (ms * 1e-3) * 1e-12 / PEAK_TFLOPS, "traffic": _traffic_bytes(),
+                     "frac": flops / (ms * 1e-3) * 1e-12 / PEAK_TFLOPS,
+                     "traffic": traffic, "traffic_source": ("from_profile: " + TRAFFIC_PROFILE) if traffic else None,
                      "flops_per_launch": flops, "algorithmic_bytes_per_launch": lib.bytes(M, N, K),
-                     "launch_ms": ms, "timer": "hipEvent pair on the null stream around the timed launches"},
+                     "launch_ms": ms, "timer": "hipEvent pair on the null stream around the timed launches",
+                     # the same work against the clock the part actually ran at during the timed launches
+                     "shader_ghz": ghz, "shader_ghz_per_xcd": [m * 1e-3 for m in clk["per_xcd_mhz"] if m > 0],
+                     "shader_ghz_min_max_over_simds": [clk["min_mhz"] * 1e-3, clk["max_mhz"] * 1e-3], "simds_sampled": clk["simds"],
+                     "nominal_ghz": NOMINAL_GHZ,
+                     "flop_per_cycle_per_cu": flop_per_cycle_per_cu,
+                     "peak_flop_per_cycle_per_cu": PEAK_FLOP_PER_CYCLE_PER_CU,
+                     "frac_at_achieved_clock": flop_per_cycle_per_cu / PEAK_FLOP_PER_CYCLE_PER_CU,
+                     "clock_source": "shader-cycle counter against the constant-rate counter, sampled on every "
+                                     "XCD before and after the timed launches"},
         "wall_ms_per_step": wall_ms,
+        "sustained": {"steps": max(args.steps, SUSTAINED_STEPS), "tflops": lib.tflops(M, N, K, sustained_ms),
+                      "ms_per_step": sustained_ms, "frac": lib.tflops(M, N, K, sustained_ms) / PEAK_TFLOPS,
+                      "shader_ghz": sustained_clk["mhz"] * 1e-3,
+                      "flop_per_cycle_per_cu": flops / (sustained_ms * 1e-3) / (sustained_clk["mhz"] * 1e6) / cus},
         "settle": {"what": "hipBLASLt launches of the same shape before the first timed leg", "calls": settle_calls,
                    "ms": settle_ms},
         "second_pass_tflops": lib.tflops(M, N, K, ms2),
-        "vendor": {"library": "hipBLASLt (fp32 compute)", "loaded_from": _loaded_library("libhipblaslt.so"),
+        "vendor": {"library": "hipBLASLt (fp32 compute)", "loaded_from": vendor.loaded_from(),
+                   **vendor.candidates(M, N, K),
                    "tflops": vendor_tflops, "ms": min(vms, vms2),
                    "first_pass_tflops": lib.tflops(M, N, K, vms), "second_pass_tflops": lib.tflops(M, N, K, vms2),
+                   "shader_ghz": vclk["mhz"] * 1e-3,
+                   "flop_per_cycle_per_cu": flops / (vms * 1e-3) / (vclk["mhz"] * 1e6) / cus,
                    "ours_over_vendor": tflops / vendor_tflops},
         "bit_identical_run_to_run": deterministic,
     }
     if not args.no_cpu:
-        cpu, chk = _cpu_baseline(torch, A, B, out)
+        cpu, chk = _cpu_baseline(A_host.view(np.uint16), B_host.view(np.uint16), out)
         result["cpu_baseline"] = cpu
         result["check_vs_cpu"] = {"rows": cpu["sample"].split(" of ")[0], "max_diff": chk["max_diff"],
                                   "rel_err": chk["rel_err"], "tolerance": chk["tol"], "ok": chk["ok"]}
@@ -195,7 +229,9 @@ def main():
     if args.sweep:
         from cuda_hgemm_amd import sweep
         os.makedirs(os.path.dirname(os.path.abspath(args.sweep_out)), exist_ok=True)
-        report = sweep.run(torch, lib, vendor, warmup=args.warmup, steps=args.steps)
+        for buf in (A, B, C, Cv):
+            buf.free()
+        report = sweep.run(lib, vendor, warmup=args.warmup, steps=args.steps)
         with open(args.sweep_out, "w") as f:
             json.dump(report, f, indent=1)
         sweep.print_table(report)

@@ -3,12 +3,14 @@
 Operand layouts are the reference's (``src/common/tester.h:117-120``): ``A`` is ``(M, K)``
 row-major, ``B`` is handed over as its ``(N, K)`` storage (column-major ``K x N``), ``C`` is
 ``(M, N)`` row-major; all fp16, all on the GPU.  Calls are asynchronous on the null stream,
-which is also torch's default stream.
+which is also torch's default stream.  Operands are torch CUDA tensors or
+``cuda_hgemm_amd.hipmem.DeviceArray`` buffers (device memory without torch).
 """
 from __future__ import annotations
 
 import ctypes as C
 import os
+import sys
 from typing import List, Optional
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -43,10 +45,14 @@ KERNEL_SYMBOLS = [
 HELPER_SYMBOLS = [
     "hgemm_auto_plan", "hgemm_auto_plan_tail", "hgemm_auto_plan_tail_kernel", "hgemm_auto_plan_chained", "hgemm_kernel_name", "hgemm_variant_count", "hgemm_variant_name", "hgemm_variant_symbol",
     "hgemm_variant_fn", "hgemm_variant_find", "hgemm_variant_supports", "hgemm_variant_in_default_run",
-    "hgemm_profile_ms", "hgemm_profile_rotating_ms", "hgemm_tflops", "hgemm_bytes", "hgemm_version",
+    "hgemm_profile_ms", "hgemm_profile_rotating_ms", "hgemm_clock_mark", "hgemm_clock_between_marks_mhz",
+    "hgemm_tflops", "hgemm_bytes", "hgemm_version",
     "hgemm_reserve_workspace", "hgemm_release_workspace", "hgemm_auto_workspace_bytes",
     "hgemm_auto_static_workspace", "hgemm_static_workspace_bytes",
 ]
+
+
+VENDOR_SYMBOLS = ["hgemm_hipblaslt", "hgemm_hipblaslt_candidates", "hgemm_hipblaslt_loaded_from"]
 
 
 def _share_hip_runtime_with_torch() -> None:
@@ -61,9 +67,16 @@ def _share_hip_runtime_with_torch() -> None:
 
 
 def _tensor_ptr(t, rows: int, cols: int, what: str) -> int:
+    from .hipmem import DeviceArray
+    if isinstance(t, DeviceArray):
+        if tuple(t.shape) != (rows, cols):
+            raise ValueError(f"{what}: expected shape {(rows, cols)}, got {tuple(t.shape)}")
+        if not t.ptr:
+            raise ValueError(f"{what}: the buffer has been freed")
+        return t.ptr
     import torch
     if not isinstance(t, torch.Tensor):
-        raise TypeError(f"{what}: expected a torch.Tensor, got {type(t).__name__}")
+        raise TypeError(f"{what}: expected a torch.Tensor or a hipmem.DeviceArray, got {type(t).__name__}")
     if t.dtype != torch.float16:
         raise TypeError(f"{what}: expected float16, got {t.dtype}")
     if not t.is_cuda:
@@ -80,13 +93,17 @@ def _tensor_ptr(t, rows: int, cols: int, what: str) -> int:
 class HgemmLibrary:
     """``libhgemm.so`` loaded through ctypes; fails loudly when it has not been built."""
 
-    def __init__(self, path: Optional[str] = None):
+    def __init__(self, path: Optional[str] = None, torch_runtime: bool = True):
+        """``torch_runtime=False``: do not import torch first, i.e. run on the system's ROCm
+        libraries (operands are then ``hipmem.DeviceArray`` buffers; importing torch later in
+        such a process would hand torch a runtime it was not built with)."""
         self.path = path or lib_path()
         if not os.path.exists(self.path):
             raise FileNotFoundError(
                 f"{self.path} is missing: build it with `python -m cuda_hgemm_amd.build` (needs hipcc); "
                 "there is no non-HIP fallback")
-        _share_hip_runtime_with_torch()
+        if torch_runtime:
+            _share_hip_runtime_with_torch()
         self.dll = C.CDLL(self.path)
         d = self.dll
         for name in KERNEL_SYMBOLS:
@@ -109,6 +126,10 @@ class HgemmLibrary:
         d.hgemm_profile_rotating_ms.argtypes = [HGEMM_FN, C.POINTER(_PTR), C.POINTER(_PTR), C.POINTER(_PTR), _SZ, _SZ,
                                                 _SZ, _SZ, _SZ, _SZ]
         d.hgemm_profile_rotating_ms.restype = C.c_double
+        d.hgemm_clock_mark.argtypes, d.hgemm_clock_mark.restype = [C.c_int], None
+        d.hgemm_clock_between_marks_mhz.argtypes = [C.POINTER(C.c_double), C.c_int, C.POINTER(C.c_double),
+                                                    C.POINTER(C.c_double)]
+        d.hgemm_clock_between_marks_mhz.restype = C.c_double
         d.hgemm_tflops.argtypes, d.hgemm_tflops.restype = [_SZ, _SZ, _SZ, C.c_double], C.c_double
         d.hgemm_bytes.argtypes, d.hgemm_bytes.restype = [_SZ, _SZ, _SZ], C.c_double
         d.hgemm_version.argtypes, d.hgemm_version.restype = [], C.c_char_p
@@ -203,6 +224,19 @@ class HgemmLibrary:
     def variant_fn(self, name: str):
         return self.dll.hgemm_variant_fn(self.find(name))
 
+    def clock_mark(self, which: int) -> None:
+        """Enqueue shader-clock sample 0 or 1 on the null stream."""
+        self.dll.hgemm_clock_mark(which)
+
+    def clock_between_marks(self, xcds: int = 8) -> dict:
+        """Average shader clock between the two marks (waits for the device)."""
+        per_xcd = (C.c_double * xcds)()
+        detail = (C.c_double * 3)()
+        elapsed = C.c_double(0.0)
+        mhz = self.dll.hgemm_clock_between_marks_mhz(per_xcd, xcds, C.byref(elapsed), detail)
+        return {"mhz": mhz, "per_xcd_mhz": list(per_xcd), "elapsed_ms": elapsed.value, "min_mhz": detail[0],
+                "max_mhz": detail[1], "simds": int(detail[2])}
+
     def tflops(self, M: int, N: int, K: int, ms: float) -> float:
         return self.dll.hgemm_tflops(M, N, K, ms)
 
@@ -213,13 +247,32 @@ class HgemmLibrary:
 class VendorLibrary:
     """``libhgemm_hipblaslt.so``: the hipBLASLt comparator, timed beside the kernels only."""
 
-    def __init__(self, path: Optional[str] = None):
+    def __init__(self, path: Optional[str] = None, torch_runtime: bool = True):
+        """``torch_runtime=False``: bind to the system's hipBLASLt instead of the copy a PyTorch
+        wheel carries under the same soname (torch must then not have been imported)."""
         self.path = path or vendor_lib_path()
         if not os.path.exists(self.path):
             raise FileNotFoundError(f"{self.path} is missing: build it with `python -m cuda_hgemm_amd.build`")
-        _share_hip_runtime_with_torch()
+        if torch_runtime:
+            _share_hip_runtime_with_torch()
+        elif "torch" in sys.modules:
+            raise RuntimeError("torch is already imported: its libhipblaslt answers the comparator's dependency")
         self.dll = C.CDLL(self.path)
         self.dll.hgemm_hipblaslt.argtypes, self.dll.hgemm_hipblaslt.restype = _HGEMM_ARGS, None
+        self.dll.hgemm_hipblaslt_candidates.argtypes = [_SZ, _SZ, _SZ, C.POINTER(C.c_int), C.POINTER(C.c_float),
+                                                        C.POINTER(C.c_float)]
+        self.dll.hgemm_hipblaslt_candidates.restype = C.c_int
+        self.dll.hgemm_hipblaslt_loaded_from.argtypes, self.dll.hgemm_hipblaslt_loaded_from.restype = [], C.c_char_p
+
+    def loaded_from(self) -> str:
+        """The hipBLASLt shared object this process bound the comparator to."""
+        return os.path.realpath(self.dll.hgemm_hipblaslt_loaded_from().decode())
+
+    def candidates(self, M: int, N: int, K: int) -> dict:
+        """What the comparator's first call for the shape found (zero candidates: not called yet)."""
+        chosen, chosen_ms, first_ms = C.c_int(-1), C.c_float(0.0), C.c_float(0.0)
+        n = self.dll.hgemm_hipblaslt_candidates(M, N, K, C.byref(chosen), C.byref(chosen_ms), C.byref(first_ms))
+        return {"candidates": n, "chosen": chosen.value, "chosen_ms": chosen_ms.value, "first_ms": first_ms.value}
 
     def fn(self):
         return C.cast(self.dll.hgemm_hipblaslt, HGEMM_FN)
@@ -233,17 +286,17 @@ _library: Optional[HgemmLibrary] = None
 _vendor: Optional[VendorLibrary] = None
 
 
-def library() -> HgemmLibrary:
+def library(torch_runtime: bool = True) -> HgemmLibrary:
     global _library
     if _library is None:
-        _library = HgemmLibrary()
+        _library = HgemmLibrary(torch_runtime=torch_runtime)
     return _library
 
 
-def vendor_library() -> VendorLibrary:
+def vendor_library(torch_runtime: bool = True) -> VendorLibrary:
     global _vendor
     if _vendor is None:
-        _vendor = VendorLibrary()
+        _vendor = VendorLibrary(torch_runtime=torch_runtime)
     return _vendor
 
 

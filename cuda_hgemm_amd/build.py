@@ -152,7 +152,7 @@ def build(force: bool = False, verbose: bool = False) -> dict:
         _run([HIPCC, "-shared", "-o", libhgemm] + lib_objs)
     ven_objs = [objs[s] for s in VENDOR_SOURCES]
     if force or _stale(vendor, ven_objs):
-        _run([HIPCC, "-shared", "-o", vendor] + ven_objs + ["-lhipblaslt"])
+        _run([HIPCC, "-shared", "-o", vendor] + ven_objs + ["-L/opt/rocm/lib", "-lhipblaslt", "-ldl", "-Wl,-rpath,/opt/rocm/lib"])
     drv_objs = [objs[s] for s in DRIVER_SOURCES]
     if force or _stale(driver, drv_objs + [libhgemm, vendor]):
         _run([HIPCC, "-o", driver] + drv_objs + ["-L" + LIB, "-lhgemm", "-lhgemm_hipblaslt", "-fopenmp",

@@ -3,6 +3,8 @@
 #include "common.h"
 #include "variant_def.h"
 
+#include <mutex>
+
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_base);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_padding);
 HGEMM_DECLARE_SUPPORTS(hgemm_mfma_swizzle);
@@ -135,6 +137,98 @@ extern "C" double hgemm_profile_rotating_ms(hgemm_fn fn, const hgemm_half *const
     HGEMM_CHECK_HIP_ERROR(hipEventDestroy(start));
     HGEMM_CHECK_HIP_ERROR(hipEventDestroy(stop));
     return (double)ms / (double)iterations;
+}
+
+// ---- shader clock between two points of the null stream.  A power-managed part runs matrix
+// work well below its nominal clock, by an amount that differs from board to board, so a
+// throughput figure is only comparable across boards together with the clock it was reached
+// at.  s_memtime counts shader cycles, s_memrealtime counts at a constant rate
+// (hipDeviceAttributeWallClockRate).  The cycle counters of different SIMDs do not share a
+// starting point (measured: tens of millions of cycles apart), so a pair of samples is only
+// meaningful when both were taken on the same SIMD of the same CU: a mark is a launch of many
+// small workgroups in which every wave files its sample under its hardware position, and the
+// clock is taken from the positions that were sampled at both marks.
+namespace {
+
+// position = XCC_ID (4 bits) | SE_ID (3) | SH_ID (1) | CU_ID (4) | SIMD_ID (2)
+constexpr int CLOCK_POSITIONS = 1 << 14, CLOCK_XCDS = 16;
+struct ClockSample {
+    unsigned long long shader, constant_rate;
+};
+std::mutex g_clock_mutex;
+ClockSample *g_clock_samples[64];  // per device: [2][CLOCK_POSITIONS], allocated by the first mark
+
+__global__ void __launch_bounds__(256) clock_clear_kernel(ClockSample *all) {
+    typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+    u64x2 zero = {0ull, 0ull};
+    *reinterpret_cast<u64x2 *>(&all[(size_t)blockIdx.x * blockDim.x + threadIdx.x]) = zero;
+}
+
+__global__ void __launch_bounds__(256) clock_mark_kernel(ClockSample *out) {
+    if ((threadIdx.x & 63) != 0) return;
+    const unsigned hw = __builtin_amdgcn_s_getreg((31 << 11) | 4);    // HW_ID: simd [5:4], cu [11:8], sh [12], se [15:13]
+    const unsigned xcc = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID [3:0]
+    const unsigned position = ((xcc & 15) << 10) | (((hw >> 13) & 7) << 7) | (((hw >> 12) & 1) << 6) |
+                              (((hw >> 8) & 15) << 2) | ((hw >> 4) & 3);
+    typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+    u64x2 v;
+    v[0] = (unsigned long long)clock64();       // s_memtime
+    v[1] = (unsigned long long)wall_clock64();  // s_memrealtime
+    *reinterpret_cast<u64x2 *>(&out[position]) = v;  // one 16-byte store: a slot never mixes two waves' samples
+}
+
+ClockSample *clock_buffer() {
+    int dev = 0;
+    HGEMM_CHECK_HIP_ERROR(hipGetDevice(&dev));
+    HGEMM_CHECK(dev >= 0 && dev < 64);
+    std::lock_guard<std::mutex> lock(g_clock_mutex);
+    if (!g_clock_samples[dev])
+        HGEMM_CHECK_HIP_ERROR(hipMalloc(reinterpret_cast<void **>(&g_clock_samples[dev]),
+                                        sizeof(ClockSample) * 2 * CLOCK_POSITIONS));
+    return g_clock_samples[dev];
+}
+
+}  // namespace
+
+extern "C" void hgemm_clock_mark(int which) {
+    HGEMM_CHECK_MSG(which == 0 || which == 1, "mark %d: there are marks 0 and 1", which);
+    ClockSample *base = clock_buffer();
+    if (which == 0)  // a position that mark 1 does not reach must not pair with a stale sample
+        clock_clear_kernel<<<dim3(2 * CLOCK_POSITIONS / 256), dim3(256), 0, nullptr>>>(base);
+    // four waves per workgroup, one per SIMD; 4096 workgroups reach every SIMD of the chip several times over
+    clock_mark_kernel<<<dim3(4096), dim3(256), 0, nullptr>>>(base + which * CLOCK_POSITIONS);
+    HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+}
+
+extern "C" double hgemm_clock_between_marks_mhz(double *per_xcd_mhz, int xcds, double *elapsed_ms, double *detail) {
+    static ClockSample h[2][CLOCK_POSITIONS];
+    static std::mutex host_mutex;
+    std::lock_guard<std::mutex> host_lock(host_mutex);
+    HGEMM_CHECK_HIP_ERROR(hipMemcpy(h, clock_buffer(), sizeof(h), hipMemcpyDeviceToHost));  // waits for the null stream
+    int dev = 0, wall_khz = 0;
+    HGEMM_CHECK_HIP_ERROR(hipGetDevice(&dev));
+    HGEMM_CHECK_HIP_ERROR(hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, dev));
+    HGEMM_CHECK_GT(wall_khz, 0);
+    double sum_mhz = 0.0, sum_ms = 0.0, lo = 0.0, hi = 0.0, xcd_sum[CLOCK_XCDS] = {};
+    int pairs = 0, xcd_pairs[CLOCK_XCDS] = {};
+    for (int p = 0; p < CLOCK_POSITIONS; ++p) {
+        if (h[0][p].constant_rate == 0 || h[1][p].constant_rate <= h[0][p].constant_rate) continue;
+        const double ticks = (double)(h[1][p].constant_rate - h[0][p].constant_rate);
+        const double mhz = (double)(h[1][p].shader - h[0][p].shader) / ticks * (double)wall_khz * 1e-3;
+        sum_mhz += mhz;
+        sum_ms += ticks / (double)wall_khz;
+        lo = (pairs == 0 || mhz < lo) ? mhz : lo;
+        hi = (pairs == 0 || mhz > hi) ? mhz : hi;
+        xcd_sum[p >> 10] += mhz;
+        ++xcd_pairs[p >> 10];
+        ++pairs;
+    }
+    HGEMM_CHECK_MSG(pairs > 0, "no SIMD was sampled at both marks: call hgemm_clock_mark(0), then (1), first");
+    for (int x = 0; per_xcd_mhz && x < xcds; ++x)
+        per_xcd_mhz[x] = (x < CLOCK_XCDS && xcd_pairs[x]) ? xcd_sum[x] / xcd_pairs[x] : 0.0;
+    if (elapsed_ms) *elapsed_ms = sum_ms / pairs;
+    if (detail) detail[0] = lo, detail[1] = hi, detail[2] = (double)pairs;
+    return sum_mhz / pairs;
 }
 
 extern "C" double hgemm_tflops(size_t M, size_t N, size_t K, double ms) {

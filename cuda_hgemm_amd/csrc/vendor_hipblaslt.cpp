@@ -3,9 +3,16 @@
 // same operand view of the row-major / column-major buffers, alpha = 1, beta = 0.
 // hipBLASLt offers no fp16-accumulate compute type, so the product is computed in fp32,
 // which is also what the hand-written kernels do.
+//
+// hipBLASLt's heuristic returns a ranked list of kernels whose first entry is often not the
+// fastest.  A 100 % line is only worth comparing against when it is the library's best, so
+// the first call for a shape asks for up to 16 candidates, times each on the caller's own
+// operands (C is overwritten by the real call that follows) and keeps the fastest.
+#include <dlfcn.h>
 #include <hipblaslt/hipblaslt.h>
 
 #include <map>
+#include <mutex>
 #include <tuple>
 
 #include "../../include/hgemm_hipblaslt.h"
@@ -23,29 +30,46 @@
 namespace {
 
 constexpr size_t kWorkspaceBytes = 128ull << 20;
+constexpr int kMaxCandidates = 16;
+constexpr int kTrialWarmup = 1, kTrialRuns = 3;
 
 struct Plan {
     hipblasLtMatmulDesc_t desc = nullptr;
     hipblasLtMatrixLayout_t layout_b = nullptr, layout_a = nullptr, layout_c = nullptr;
     hipblasLtMatmulAlgo_t algo;
-    size_t workspace = 0;
+    int candidates = 0, chosen = -1;  // how many kernels the heuristic offered, and which one was fastest
+    float chosen_ms = 0.f, first_ms = 0.f;
 };
+
+// Plans by shape.  Kept apart from the handle so that asking what is known about a shape
+// touches neither the GPU nor hipBLASLt.
+std::mutex g_plans_mutex;
+std::map<std::tuple<size_t, size_t, size_t>, Plan> g_plans;
+
+const Plan *find_plan(size_t M, size_t N, size_t K) {  // caller holds g_plans_mutex
+    auto it = g_plans.find(std::make_tuple(M, N, K));
+    return it == g_plans.end() ? nullptr : &it->second;
+}
 
 struct Context {
     hipblasLtHandle_t handle = nullptr;
     void *workspace = nullptr;
-    std::map<std::tuple<size_t, size_t, size_t>, Plan> plans;
 
     Context() {
         HGEMM_CHECK_HIPBLASLT_ERROR(hipblasLtCreate(&handle));
         HGEMM_CHECK_HIP_ERROR(hipMalloc(&workspace, kWorkspaceBytes));
     }
 
+    hipblasStatus_t run(const Plan &p, const hipblasLtMatmulAlgo_t &algo, const void *A, const void *B, void *C) {
+        static const float alpha = 1.0f, beta = 0.0f;
+        return hipblasLtMatmul(handle, p.desc, &alpha, B, p.layout_b, A, p.layout_a, &beta, C, p.layout_c, C,
+                               p.layout_c, &algo, workspace, kWorkspaceBytes, nullptr);
+    }
+
     // Column-major view: C^T (N x M, ld N) = op_T(B as K x N, ld K) * (A as K x M, ld K).
-    const Plan &plan_for(size_t M, size_t N, size_t K) {
-        auto key = std::make_tuple(M, N, K);
-        auto it = plans.find(key);
-        if (it != plans.end()) return it->second;
+    const Plan &plan_for(const void *A, const void *B, void *C, size_t M, size_t N, size_t K) {
+        std::lock_guard<std::mutex> lock(g_plans_mutex);
+        if (const Plan *known = find_plan(M, N, K)) return *known;
         Plan p;
         HGEMM_CHECK_HIPBLASLT_ERROR(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
         hipblasOperation_t op_t = HIPBLAS_OP_T, op_n = HIPBLAS_OP_N;
@@ -61,27 +85,75 @@ struct Context {
         size_t ws = kWorkspaceBytes;
         HGEMM_CHECK_HIPBLASLT_ERROR(hipblasLtMatmulPreferenceSetAttribute(
             pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws)));
-        hipblasLtMatmulHeuristicResult_t result[1];
+        hipblasLtMatmulHeuristicResult_t result[kMaxCandidates];
         int found = 0;
         HGEMM_CHECK_HIPBLASLT_ERROR(hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.layout_b, p.layout_a, p.layout_c,
-                                                                    p.layout_c, pref, 1, result, &found));
+                                                                    p.layout_c, pref, kMaxCandidates, result, &found));
         HGEMM_CHECK_MSG(found > 0, "hipBLASLt has no algorithm for M=%zu N=%zu K=%zu", M, N, K);
-        p.algo = result[0].algo;
-        p.workspace = result[0].workspaceSize;
         HGEMM_CHECK_HIPBLASLT_ERROR(hipblasLtMatmulPreferenceDestroy(pref));
-        return plans.emplace(key, p).first->second;
+        p.candidates = found;
+
+        // Time every candidate: a warm-up call, then kTrialRuns calls between two events.
+        hipEvent_t start = nullptr, stop = nullptr;
+        HGEMM_CHECK_HIP_ERROR(hipEventCreate(&start));
+        HGEMM_CHECK_HIP_ERROR(hipEventCreate(&stop));
+        for (int c = 0; c < found; ++c) {
+            if (result[c].state != HIPBLAS_STATUS_SUCCESS || result[c].workspaceSize > kWorkspaceBytes) continue;
+            bool ok = true;
+            for (int i = 0; i < kTrialWarmup && ok; ++i) ok = run(p, result[c].algo, A, B, C) == HIPBLAS_STATUS_SUCCESS;
+            if (!ok) continue;
+            HGEMM_CHECK_HIP_ERROR(hipEventRecord(start, nullptr));
+            for (int i = 0; i < kTrialRuns && ok; ++i) ok = run(p, result[c].algo, A, B, C) == HIPBLAS_STATUS_SUCCESS;
+            HGEMM_CHECK_HIP_ERROR(hipEventRecord(stop, nullptr));
+            HGEMM_CHECK_HIP_ERROR(hipEventSynchronize(stop));
+            if (!ok) continue;
+            float ms = 0.f;
+            HGEMM_CHECK_HIP_ERROR(hipEventElapsedTime(&ms, start, stop));
+            ms /= (float)kTrialRuns;
+            if (c == 0) p.first_ms = ms;
+            if (p.chosen < 0 || ms < p.chosen_ms) {
+                p.chosen = c;
+                p.chosen_ms = ms;
+                p.algo = result[c].algo;
+            }
+        }
+        HGEMM_CHECK_HIP_ERROR(hipEventDestroy(start));
+        HGEMM_CHECK_HIP_ERROR(hipEventDestroy(stop));
+        HGEMM_CHECK_MSG(p.chosen >= 0, "none of hipBLASLt's %d candidates ran for M=%zu N=%zu K=%zu", found, M, N, K);
+        return g_plans.emplace(std::make_tuple(M, N, K), p).first->second;
     }
 };
+
+Context &context() {
+    static Context ctx;
+    return ctx;
+}
 
 }  // namespace
 
 extern "C" void hgemm_hipblaslt(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N,
                                 size_t K) {
     hgemm::check_operands(A, B, C, M, N, K);
-    static Context ctx;
-    static const float alpha = 1.0f, beta = 0.0f;
-    const Plan &p = ctx.plan_for(M, N, K);
-    HGEMM_CHECK_HIPBLASLT_ERROR(hipblasLtMatmul(ctx.handle, p.desc, &alpha, B, p.layout_b, A, p.layout_a, &beta, C,
-                                                p.layout_c, C, p.layout_c, &p.algo, ctx.workspace, kWorkspaceBytes,
-                                                nullptr));
+    Context &ctx = context();
+    const Plan &p = ctx.plan_for(A, B, C, M, N, K);
+    HGEMM_CHECK_HIPBLASLT_ERROR(ctx.run(p, p.algo, A, B, C));
+}
+
+extern "C" int hgemm_hipblaslt_candidates(size_t M, size_t N, size_t K, int *chosen, float *chosen_ms,
+                                          float *first_ms) {
+    std::lock_guard<std::mutex> lock(g_plans_mutex);
+    const Plan *p = find_plan(M, N, K);
+    if (!p) return 0;
+    if (chosen) *chosen = p->chosen;
+    if (chosen_ms) *chosen_ms = p->chosen_ms;
+    if (first_ms) *first_ms = p->first_ms;
+    return p->candidates;
+}
+
+extern "C" const char *hgemm_hipblaslt_loaded_from(void) {
+    static char path[1024] = "";
+    Dl_info info;
+    if (path[0] == 0 && dladdr(reinterpret_cast<const void *>(&hipblasLtMatmul), &info) && info.dli_fname)
+        snprintf(path, sizeof(path), "%s", info.dli_fname);
+    return path;
 }

@@ -15,16 +15,23 @@ DECODE_M = [1, 8, 16, 64, 128]
 DECODE_NK = [(4096, 4096), (28672, 4096)]
 
 
-def _draw(torch, dev, gen, rows, cols, dist):
-    if dist == "uniform":
-        return (torch.rand((rows, cols), device=dev, generator=gen, dtype=torch.float32) * 2.0 - 1.0).half()
-    sigma = {"normal": 1.0, "weights": 0.02}[dist]
-    return (torch.randn((rows, cols), device=dev, generator=gen, dtype=torch.float32) * sigma).half()
+def _draw(rng, rows, cols, dist):
+    """fp16 matrix on the host: uniform[-1,1), or normal(0, sigma) with sigma 1 (activations) or 0.02 (weights)."""
+    import numpy as np
+    out = np.empty((rows, cols), np.float16)
+    step = max(1, (1 << 24) // cols)
+    for r in range(0, rows, step):  # in slabs: no full-size fp32 temporary
+        shape = (min(step, rows - r), cols)
+        if dist == "uniform":
+            out[r:r + step] = rng.random(shape, dtype=np.float32) * 2.0 - 1.0
+        else:
+            out[r:r + step] = rng.standard_normal(shape, dtype=np.float32) * {"normal": 1.0, "weights": 0.02}[dist]
+    return out
 
 
-def _time(torch, lib, fn, As, Bs, Cs, m, n, k, warmup, steps):
+def _time(hipmem, lib, fn, As, Bs, Cs, m, n, k, warmup, steps):
     lib.profile_fn_rotating_ms(fn, As, Bs, Cs, m, n, k, 0, warmup)
-    torch.cuda.synchronize()
+    hipmem.synchronize()
     return lib.profile_fn_rotating_ms(fn, As, Bs, Cs, m, n, k, 0, steps)
 
 
@@ -42,40 +49,50 @@ def _row(lib, kind, m, n, k, ms, vms, extra=None):
     return row
 
 
-def run(torch, lib, vendor, warmup=10, steps=100):
-    dev = torch.device("cuda:0")
-    gen = torch.Generator(device=dev).manual_seed(20230212)
+def run(lib, vendor, warmup=10, steps=100):
+    """Every size with `warmup` untimed and `steps` timed launches, the vendor GEMM first."""
+    import numpy as np
+    from . import hipmem
+    dev_array = hipmem.DeviceArray
+    rng = np.random.default_rng(20230212)
     auto, vfn = lib.variant_fn("hgemm_auto"), vendor.fn()
     rows = []
+
+    def one(kind, m, n, k, dist_a, dist_b):
+        A, B = dev_array.from_host(_draw(rng, m, k, dist_a)), dev_array.from_host(_draw(rng, n, k, dist_b))
+        C = dev_array((m, n))
+        vms = _time(hipmem, lib, vfn, [A], [B], [C], m, n, k, warmup, steps)
+        ms = _time(hipmem, lib, auto, [A], [B], [C], m, n, k, warmup, steps)
+        rows.append(_row(lib, kind, m, n, k, ms, vms, {"vendor_pick": vendor.candidates(m, n, k)}))
+        for buf in (A, B, C):
+            buf.free()
+
     for s in SQUARES:
-        A, B = _draw(torch, dev, gen, s, s, "uniform"), _draw(torch, dev, gen, s, s, "uniform")
-        C = torch.empty((s, s), dtype=torch.float16, device=dev)
-        it = steps if s < 16384 else max(10, steps // 5)
-        vms = _time(torch, lib, vfn, [A], [B], [C], s, s, s, warmup, it)
-        ms = _time(torch, lib, auto, [A], [B], [C], s, s, s, warmup, it)
-        rows.append(_row(lib, "square", s, s, s, ms, vms))
-        del A, B, C
+        one("square", s, s, s, "uniform", "uniform")
     for (m, n, k) in FFN:
-        A, B = _draw(torch, dev, gen, m, k, "uniform"), _draw(torch, dev, gen, n, k, "weights")
-        C = torch.empty((m, n), dtype=torch.float16, device=dev)
-        vms = _time(torch, lib, vfn, [A], [B], [C], m, n, k, warmup, steps)
-        ms = _time(torch, lib, auto, [A], [B], [C], m, n, k, warmup, steps)
-        rows.append(_row(lib, "ffn", m, n, k, ms, vms))
-        del A, B, C
+        one("ffn", m, n, k, "uniform", "weights")
     for (n, k) in DECODE_NK:
         copies = max(2, (768 << 20) // (n * k * 2) + 1)   # > 3x the 256 MB Infinity Cache in total
-        Bs = [_draw(torch, dev, gen, n, k, "weights") for _ in range(copies)]
+        base = _draw(rng, n, k, "weights")
+        # distinct buffers are what matters (every call must stream its B from HBM), not distinct values:
+        # copy i is the same draw with its rows rotated by i
+        Bs = [dev_array.from_host(np.roll(base, i, axis=0)) for i in range(copies)]
         for m in DECODE_M:
-            As = [_draw(torch, dev, gen, m, k, "normal") for _ in range(copies)]
-            Cs = [torch.empty((m, n), dtype=torch.float16, device=dev) for _ in range(copies)]
-            warm_ms = _time(torch, lib, auto, As[:1], Bs[:1], Cs[:1], m, n, k, warmup, steps)
-            cold_ms = _time(torch, lib, auto, As, Bs, Cs, m, n, k, warmup, steps)
-            vcold_ms = _time(torch, lib, vfn, As, Bs, Cs, m, n, k, warmup, steps)
+            a_base = _draw(rng, m, k, "normal")
+            As = [dev_array.from_host(np.roll(a_base, i, axis=1)) for i in range(copies)]
+            Cs = [dev_array((m, n)) for _ in range(copies)]
+            warm_ms = _time(hipmem, lib, auto, As[:1], Bs[:1], Cs[:1], m, n, k, warmup, steps)
+            cold_ms = _time(hipmem, lib, auto, As, Bs, Cs, m, n, k, warmup, steps)
+            vcold_ms = _time(hipmem, lib, vfn, As, Bs, Cs, m, n, k, warmup, steps)
             rows.append(_row(lib, "decode", m, n, k, cold_ms, vcold_ms,
                              {"cache_warm_ms": warm_ms, "cache_warm_gbps": lib.bytes(m, n, k) / (warm_ms * 1e-3) * 1e-9,
-                              "operand_sets": copies}))
-        del Bs
-    return {"peak_tflops": PEAK_TFLOPS, "peak_gbps": PEAK_GBPS, "warmup": warmup, "steps": steps, "rows": rows}
+                              "operand_sets": copies, "vendor_pick": vendor.candidates(m, n, k)}))
+            for buf in As + Cs:
+                buf.free()
+        for buf in Bs:
+            buf.free()
+    return {"peak_tflops": PEAK_TFLOPS, "peak_gbps": PEAK_GBPS, "warmup": warmup, "steps": steps,
+            "vendor_loaded_from": vendor.loaded_from(), "rows": rows}
 
 
 def print_table(report, file=None):

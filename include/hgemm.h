@@ -211,6 +211,20 @@ double hgemm_profile_ms(hgemm_fn fn, const hgemm_half *A, const hgemm_half *B, h
 double hgemm_profile_rotating_ms(hgemm_fn fn, const hgemm_half *const *A, const hgemm_half *const *B,
                                  hgemm_half *const *C, size_t n_sets, size_t M, size_t N, size_t K, size_t warmup,
                                  size_t iterations);
+/* Shader clock sustained between two points of the null stream (no counterpart in the
+ * reference, whose hardware held its clock: on a power-managed part the clock under matrix
+ * load differs from board to board, and throughput is only comparable together with it).
+ * hgemm_clock_mark(0) and hgemm_clock_mark(1) each enqueue a small kernel whose waves sample
+ * the shader-cycle counter and the constant-rate counter and file the pair under the SIMD
+ * they run on (the first mark on a device allocates the 512 KB the samples live in).
+ * hgemm_clock_between_marks_mhz waits for the device and returns the average shader clock in
+ * MHz between the marks, taken over the SIMDs that were sampled at both; per XCD into
+ * per_xcd_mhz[0 .. xcds) if not NULL (0 for an XCD without such a SIMD); through elapsed_ms
+ * if not NULL the time between the marks by the constant-rate counter; through detail if not
+ * NULL three numbers: the lowest and the highest clock of a single SIMD, and how many SIMDs
+ * were used. */
+void hgemm_clock_mark(int which);
+double hgemm_clock_between_marks_mhz(double *per_xcd_mhz, int xcds, double *elapsed_ms, double *detail);
 /* 2*M*N*K*1e-12 / (ms*1e-3)  (reference src/common/tester.h:96-97). */
 double hgemm_tflops(size_t M, size_t N, size_t K, double ms);
 /* Algorithmic bytes of one call: 2*(M*K + K*N + M*N). */

@@ -16,7 +16,19 @@
 extern "C" {
 #endif
 
+/* The first call for a shape asks hipBLASLt's heuristic for up to 16 kernels, times each on
+ * the caller's operands (one warm-up and three timed calls: C is overwritten) and keeps the
+ * fastest, so that the 100 % line is the library's best kernel and not merely its first guess;
+ * later calls of that shape go straight to the kept kernel. */
 HGEMM_FUNC(hgemm_hipblaslt);
+
+/* What that first call found for a shape: the number of kernels the heuristic offered (0 if
+ * the shape has not been called yet) and, through the pointers that are not NULL, the index
+ * of the fastest, its time and the time of the heuristic's first entry (ms per call). */
+int hgemm_hipblaslt_candidates(size_t M, size_t N, size_t K, int *chosen, float *chosen_ms, float *first_ms);
+
+/* Path of the hipBLASLt shared object this comparator is bound to in this process. */
+const char *hgemm_hipblaslt_loaded_from(void);
 
 #ifdef __cplusplus
 }

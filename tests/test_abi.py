@@ -32,9 +32,15 @@ def test_library_exports_every_declared_symbol(hgemm_lib):
     assert declared == set(KERNEL_SYMBOLS) | set(HELPER_SYMBOLS)
 
 
-def test_vendor_library_exports_its_symbol(vendor_lib):
-    assert _declared_symbols("hgemm_hipblaslt.h") == {"hgemm_hipblaslt"}
-    assert hasattr(vendor_lib.dll, "hgemm_hipblaslt")
+def test_vendor_library_exports_its_symbols(vendor_lib):
+    from cuda_hgemm_amd.binding import VENDOR_SYMBOLS
+    declared = _declared_symbols("hgemm_hipblaslt.h")
+    assert declared == set(VENDOR_SYMBOLS) and "hgemm_hipblaslt" in declared
+    for name in sorted(declared):
+        assert hasattr(vendor_lib.dll, name), f"libhgemm_hipblaslt.so does not export {name}"
+    # bound to a hipBLASLt that exists; a shape that has not been called has no candidates yet (no GPU call here)
+    assert os.path.exists(vendor_lib.loaded_from()) and "hipblaslt" in vendor_lib.loaded_from().lower()
+    assert vendor_lib.candidates(123, 456, 789)["candidates"] == 0
 
 
 def test_measured_library_has_no_blas_dependency(hgemm_lib):

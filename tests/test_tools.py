@@ -90,3 +90,45 @@ def test_parse_and_tables(tmp_path):
 
 def test_empty_directory_is_an_error(tmp_path):
     assert performance.analyze(str(tmp_path)) == 1
+
+
+# ------------------------------------------------------------------ the build's resource guard
+def _remarks(kernels):
+    lines = []
+    for name, (vgprs, agprs, scratch, spill) in kernels.items():
+        tag = "x.hip:1:1: remark: "
+        lines += [tag + f"Function Name: {name} [-Rpass-analysis=kernel-resource-usage]",
+                  tag + "    SGPRs: 40 [-Rpass-analysis=kernel-resource-usage]",
+                  tag + f"    VGPRs: {vgprs} [-Rpass-analysis=kernel-resource-usage]",
+                  tag + f"    AGPRs: {agprs} [-Rpass-analysis=kernel-resource-usage]",
+                  tag + f"    ScratchSize [bytes/lane]: {scratch} [-Rpass-analysis=kernel-resource-usage]",
+                  tag + "    SGPRs Spill: 3 [-Rpass-analysis=kernel-resource-usage]",
+                  tag + f"    VGPRs Spill: {spill} [-Rpass-analysis=kernel-resource-usage]"]
+    return "\n".join(lines)
+
+
+def test_build_guard_for_the_inline_assembly_kernels():
+    """The build must fail when a hand-scheduled kernel spills, when a chained kernel's AGPR count is not exactly
+    its named accumulators (or its VGPRs reach 256), and when the guard finds nothing to check."""
+    import pytest
+    from cuda_hgemm_amd import build
+    chained = "_ZN5hgemm20hgemm_chained_kernelINS_10PipeConfigILi256ELi256ELi64ELi2ELi2ELi2ELi16ELi1EEELb0ELb0EEEvPKDF16_"
+    chained192 = "_ZN5hgemm20hgemm_chained_kernelINS_10PipeConfigILi192ELi192ELi64ELi2ELi2ELi3ELi16ELi0EEELb0ELb0EEEvPKDF16_"
+    piped = "_ZN5hgemm22hgemm_pipelined_kernelINS_10PipeConfigILi128ELi128ELi64ELi2ELi2ELi5ELi16ELi0EEELb0ELb0EEEvPKDF16_"
+    other = "_ZN5hgemm15pad_copy_kernelEPKDF16_PDF16_iiii"
+    assert build._chained_accumulator_registers(chained) == 256
+    assert build._chained_accumulator_registers(chained192) == 144
+    good = {chained: (179, 256, 0, 0), chained192: (139, 144, 0, 0), piped: (88, 64, 0, 0), other: (11, 0, 16, 2)}
+    assert build._check_no_spills("dispatch.hip", _remarks(good)) == {"hgemm_chained_kernel", "hgemm_pipelined_kernel"}
+    for bad in ({**good, piped: (88, 64, 8, 0)},             # scratch
+                {**good, chained: (179, 256, 0, 1)},         # a spilled VGPR
+                {**good, chained: (179, 260, 0, 0)},         # the compiler took AGPRs of its own
+                {**good, chained192: (139, 128, 0, 0)},      # fewer AGPRs than named accumulators
+                {**good, chained: (256, 256, 0, 0)},         # VGPRs exhausted
+                {other: (11, 0, 0, 0)},                      # nothing to check in a file that must have such kernels
+                {piped: (88, 64, 0, 0)}):                    # ... or only one of the two kinds
+        with pytest.raises(RuntimeError):
+            build._check_no_spills("dispatch.hip", _remarks(bad))
+    with pytest.raises(RuntimeError):                        # a remark format the parser does not understand
+        build._check_no_spills("dispatch.hip", _remarks(good).replace("VGPRs:", "ArchVGPRs:"))
+    assert build._check_no_spills("basic_kernels.hip", _remarks({other: (11, 0, 16, 2)})) == set()
