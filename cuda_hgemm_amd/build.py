@@ -130,6 +130,8 @@ def _compile(src, force):
             flags = flags + ["-Rpass-analysis=kernel-resource-usage"]
         out = _run([HIPCC] + flags + ["-c", path, "-o", obj])
         if src.endswith(".hip"):
+            with open(obj + ".resources.txt", "w") as f:  # registers, scratch and occupancy per kernel, for inspection
+                f.write(out)
             try:
                 _check_no_spills(src, out)
             except RuntimeError:

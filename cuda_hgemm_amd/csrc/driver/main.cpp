@@ -24,9 +24,9 @@ static void write_json(const std::string &path, const Tester &tester, size_t M, 
     for (size_t i = 0; i < recs.size(); ++i) {
         const EvalRecord &r = recs[i];
         fprintf(f,
-                "  {\"name\": \"%s\", \"ms\": %.6f, \"tflops\": %.3f, \"gbps\": %.1f, \"pct_of_first\": %.2f, "
+                "  {\"name\": \"%s\", \"ms\": %.6f, \"tflops\": %.3f, \"gbps\": %.1f, \"shader_mhz\": %.0f, \"pct_of_first\": %.2f, "
                 "\"checked\": %s, \"pass\": %s, \"max_diff\": %.6g, \"avg_diff\": %.6g, \"rel_err\": %.6g}%s\n",
-                r.name.c_str(), r.ms, r.tflops, r.gbps, r.pct_of_base, r.checked ? "true" : "false",
+                r.name.c_str(), r.ms, r.tflops, r.gbps, r.shader_mhz, r.pct_of_base, r.checked ? "true" : "false",
                 r.pass ? "true" : "false", r.max_diff, r.avg_diff, r.rel_err, i + 1 < recs.size() ? "," : "");
     }
     fprintf(f, " ]}\n");

@@ -25,6 +25,7 @@ namespace hgemm {
 struct EvalRecord {
     std::string name;
     double warmup_ms = 0.0, ms = 0.0, tflops = 0.0, gbps = 0.0, pct_of_base = 0.0;
+    double shader_mhz = 0.0;  // average shader clock over the timed calls
     bool checked = false, pass = true;
     double max_diff = 0.0, avg_diff = 0.0, rel_err = 0.0;
 };
@@ -46,6 +47,10 @@ public:
         HGEMM_CHECK_GT(m_warmup_iterations, 0u);
         HGEMM_CHECK_GT(m_profiling_iterations, 0u);
         HGEMM_CHECK_GT(m_sleep_duration, 0u);
+        int dev = 0;
+        HGEMM_CHECK_HIP_ERROR(hipGetDevice(&dev));
+        HGEMM_CHECK_HIP_ERROR(hipDeviceGetAttribute(&m_compute_units, hipDeviceAttributeMultiprocessorCount, dev));
+        HGEMM_CHECK_GT(m_compute_units, 0);
 
         m_A = std::make_shared<Matrix>(m_M, m_K, "Matrix A", seed, 1, fill_a);
         m_B = std::make_shared<Matrix>(m_K, m_N, "Matrix B", seed, 2, fill_b);  // stored as N rows of K
@@ -133,12 +138,15 @@ public:
 private:
     template <typename Func>
     void profile(Func &&hgemm, EvalRecord &rec) {
+        hgemm_clock_mark(0);  // the shader clock the part sustains over the timed calls (it is power-managed)
         m_timer.start();
         for (size_t i = 0; i < m_profiling_iterations; ++i) {
             const size_t s = i % m_As.size();
             hgemm(m_As[s], m_Bs[s], m_Cs[s], m_M, m_N, m_K);
         }
         rec.ms = static_cast<double>(m_timer.end()) / static_cast<double>(m_profiling_iterations);
+        hgemm_clock_mark(1);
+        rec.shader_mhz = hgemm_clock_between_marks_mhz(nullptr, 0, nullptr, nullptr);
         rec.tflops = hgemm_tflops(m_M, m_N, m_K, rec.ms);
         rec.gbps = hgemm_bytes(m_M, m_N, m_K) / (rec.ms * 1e-3) * 1e-9;
 
@@ -150,13 +158,16 @@ private:
 
         HLOG("%s exit, profiling time: %.3f ms (%.2f%%), throughput: %.3f TFLOPS (%.2f%%)", rec.name.c_str(), rec.ms,
              rec.ms / m_base_time * 100, rec.tflops, rec.pct_of_base);
-        HLOG("%s roofline: %.2f%% of 2500 TFLOPS dense FP16, %.1f GB/s algorithmic (%.2f%% of 8000 GB/s)",
-             rec.name.c_str(), rec.tflops / 2500.0 * 100, rec.gbps, rec.gbps / 8000.0 * 100);
+        HLOG("%s roofline: %.2f%% of 2500 TFLOPS dense FP16, %.1f GB/s algorithmic (%.2f%% of 8000 GB/s), shader clock "
+             "%.0f MHz: %.0f flop per cycle and CU of 4096",
+             rec.name.c_str(), rec.tflops / 2500.0 * 100, rec.gbps, rec.gbps / 8000.0 * 100, rec.shader_mhz,
+             rec.tflops * 1e12 / (rec.shader_mhz * 1e6) / (double)m_compute_units);
     }
 
     const size_t m_M, m_N, m_K;
     const size_t m_warmup_iterations, m_profiling_iterations, m_sleep_duration;
     const bool m_enable_check;
+    int m_compute_units = 0;
 
     std::shared_ptr<Matrix> m_A;     // row major, M * K
     std::shared_ptr<Matrix> m_B;     // col major, K * N

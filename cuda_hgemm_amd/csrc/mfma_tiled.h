@@ -140,8 +140,14 @@ __device__ __forceinline__ int swizzle_of_row(int row) {
 // instructions in order, so no wait is needed between a store and the load that picks the data up in another lane;
 // but the compiler reasons lane by lane: where it can prove that the bytes a lane stores and the bytes the same lane
 // loads never coincide, it is free to issue the load first (it did, for some tile shapes: stale strip contents in
-// the output).  An empty ordered statement that claims to touch memory keeps stores and loads on their own sides.
-__device__ __forceinline__ void wave_lds_exchange_point() { asm volatile("" ::: "memory"); }
+// the output).  What the exchange needs is what the language calls it: the stores released and the loads acquired
+// at wavefront scope, around a wave barrier.  None of the three emits an instruction; they keep the stores and the
+// loads on their own sides.
+__device__ __forceinline__ void wave_lds_exchange_point() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 
 // C is written once and never read back by these kernels: stored with the non-temporal hint its lines do not
 // displace the A and B panels that other workgroups are about to read from L2 and the Infinity Cache (measured on
