@@ -43,7 +43,8 @@ KERNEL_SYMBOLS = [
     "hgemm_mfma_chained_256x256", "hgemm_skinny", "hgemm_auto",
 ]
 HELPER_SYMBOLS = [
-    "hgemm_auto_plan", "hgemm_auto_plan_tail", "hgemm_auto_plan_tail_kernel", "hgemm_auto_plan_chained", "hgemm_kernel_name", "hgemm_variant_count", "hgemm_variant_name", "hgemm_variant_symbol",
+    "hgemm_auto_plan", "hgemm_auto_plan_tail", "hgemm_auto_plan_tail_kernel", "hgemm_auto_plan_chained", "hgemm_kernel_name",
+    "hgemm_small_m_rule", "hgemm_variant_count", "hgemm_variant_name", "hgemm_variant_symbol",
     "hgemm_variant_fn", "hgemm_variant_find", "hgemm_variant_supports", "hgemm_variant_in_default_run",
     "hgemm_profile_ms", "hgemm_profile_rotating_ms", "hgemm_clock_mark", "hgemm_clock_between_marks_mhz",
     "hgemm_tflops", "hgemm_bytes", "hgemm_version",
@@ -114,6 +115,8 @@ class HgemmLibrary:
         d.hgemm_auto_plan_tail_kernel.argtypes, d.hgemm_auto_plan_tail_kernel.restype = [_SZ, _SZ, _SZ], C.c_int
         d.hgemm_auto_plan_chained.argtypes, d.hgemm_auto_plan_chained.restype = [_SZ, _SZ, _SZ], C.c_int
         d.hgemm_kernel_name.argtypes, d.hgemm_kernel_name.restype = [C.c_int], C.c_char_p
+        d.hgemm_small_m_rule.argtypes = [C.c_int, C.POINTER(_SZ), C.POINTER(C.c_int)]
+        d.hgemm_small_m_rule.restype = C.c_int
         d.hgemm_variant_count.argtypes, d.hgemm_variant_count.restype = [], C.c_int
         d.hgemm_variant_name.argtypes, d.hgemm_variant_name.restype = [C.c_int], C.c_char_p
         d.hgemm_variant_symbol.argtypes, d.hgemm_variant_symbol.restype = [C.c_int], C.c_char_p
@@ -167,6 +170,20 @@ class HgemmLibrary:
                 "chained": bool(self.dll.hgemm_auto_plan_chained(M, N, K)),
                 "tail_tiles": tail_tiles, "tail_splits": tail_splits.value,
                 "tail_kernel": self.dll.hgemm_kernel_name(self.dll.hgemm_auto_plan_tail_kernel(M, N, K)).decode()}
+
+    def small_m_rules(self) -> List[dict]:
+        """The table behind hgemm_auto's choice for M <= 128, in order (first covering row wins)."""
+        rows, i = [], 0
+        while True:
+            bounds, flags = (_SZ * 8)(), C.c_int(0)
+            kernel = self.dll.hgemm_small_m_rule(i, bounds, C.byref(flags))
+            if kernel < 0:
+                return rows
+            keys = ("m_lo", "m_hi", "n_lo", "n_hi", "k_lo", "k_hi", "b_lo", "b_hi")
+            rows.append({**dict(zip(keys, list(bounds))), "k_below_4n": bool(flags.value & 1),
+                         "k_not_multiple_of_16384": bool(flags.value & 2), "kernel_id": kernel,
+                         "kernel": self.dll.hgemm_kernel_name(kernel).decode()})
+            i += 1
 
     def auto_workspace_bytes(self, M: int, N: int, K: int) -> dict:
         operands = _SZ(0)

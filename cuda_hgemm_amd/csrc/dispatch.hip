@@ -316,6 +316,91 @@ int choose_splits(size_t tiles, size_t cus, size_t K, size_t slice_bytes, size_t
     return s;
 }
 
+
+// ---- kernels for M <= 128 ("decode-shaped": B is streamed once, the bound is HBM bandwidth).  Which kernel runs
+// where was settled by timing the candidates against each other on an MI355X, operands rotated so that every call
+// reads HBM: library builds with and without a rule, hgemm_auto on both in one process, over K = 256 ... 28672 x
+// N = 256 ... 32768 x M = 1 ... 128.  The outcome is this table: the first row that covers a shape, and whose
+// kernel can run it (divisibility), decides.  Rows are boxes in (M, N, K, elements of B); the two conditions that
+// are not boxes are flags.
+enum SmallMFlags {
+    RULE_K_BELOW_4N = 1,        // only where K < 4 N (beyond, K slices across workgroups win)
+    RULE_K_NOT_16384S = 2,      // not where K is a multiple of 16384 (the ring kernel's 16 rows of B per workgroup then
+                                // lie 32 KB apart: 20-28 % behind)
+};
+struct SmallMRule {
+    int m_lo, m_hi;
+    size_t n_lo, n_hi, k_lo, k_hi, b_lo, b_hi;  // inclusive bounds; b = N * K, the elements of B
+    int flags, kernel;
+};
+constexpr size_t ANY = ~(size_t)0;
+constexpr size_t LARGE_B = (size_t)48 << 20;  // elements: a B of 96 MB
+constexpr SmallMRule SMALL_M_RULES[] = {
+    // --- M = 1 ... 8.  Below K = 1024 the streaming kernel (as fast or faster, M = 1 by 6-26 %) where it can run,
+    // i.e. N % 32 == 0 and K % 256 == 0; else the ring kernel (2.0x median over what ran such shapes before).
+    {1, 8, 1, 8192, 256, 1023, 0, ANY, 0, KERNEL_DECODE_BN16},
+    // The ring kernel: 0-60 % ahead (median 18 %) except against a B of 96 MB or more with K < 8192 (ties at M <= 8,
+    // the split-K kernel streams B past the caches there) and except K < 2048 against N > 8192 (up to 4 % behind).
+    {1, 8, 1, 8192, 256, 2047, 0, ANY, 0, KERNEL_DECODE_RING},
+    {1, 8, 1, ANY, 2048, 8191, 0, LARGE_B - 1, 0, KERNEL_DECODE_RING},
+    {1, 8, 1, ANY, 8192, ANY, 0, LARGE_B - 1, 0, KERNEL_DECODE_RING},
+    {1, 8, 1, ANY, 8192, ANY, LARGE_B, ANY, RULE_K_NOT_16384S, KERNEL_DECODE_RING},
+    // M = 6 ... 8 against a B of 96 MB or more: the split-K kernel (N = 14336: 8-16 % ahead of the streaming kernel,
+    // N = 28672: 2-3 %); below M = 6 and for smaller B the streaming kernel stays ahead.
+    {6, 8, 1, ANY, 1, ANY, LARGE_B, ANY, 0, KERNEL_SPLIT_32x64},
+    {1, 8, 1, ANY, 1, ANY, 0, ANY, 0, KERNEL_DECODE_BN16},
+    // --- M = 9 ... 16: the ring kernel up to N = 8192 while K <= 4096 (K <= 8192 up to N = 4096); beyond, K slices
+    // across workgroups are up to 29 % ahead.
+    {9, 16, 1, 8192, 256, 4096, 0, ANY, RULE_K_BELOW_4N, KERNEL_DECODE_RING},
+    {9, 16, 1, 4096, 4097, 8192, 0, ANY, RULE_K_BELOW_4N, KERNEL_DECODE_RING},
+    // --- M = 17 ... 64 (two or four row tiles of A per wave): the ring kernel while K is short, where one launch beats
+    // the split-K kernel plus the launch that adds its slices: K < 1024 up to N = 8192 (median 1.65x), K <= 2048 up
+    // to N = 4096 (median 1.31x); and up to K = 4096 for M <= 24 against N = 3072 ... 4096 (median 1.21x; at
+    // N <= 2048 M = 24 is 1-9 % behind).
+    {17, 64, 1, 8192, 256, 1023, 0, ANY, RULE_K_BELOW_4N, KERNEL_DECODE_RING},
+    {17, 64, 1, 4096, 1024, 2048, 0, ANY, RULE_K_BELOW_4N, KERNEL_DECODE_RING},
+    {17, 24, 3072, 4096, 2049, 4096, 0, ANY, RULE_K_BELOW_4N, KERNEL_DECODE_RING},
+    // --- M = 65 ... 128 (eight row tiles): the ring kernel for K <= 512 up to N = 8192, K <= 1024 up to N = 4096
+    // (median 1.45x).
+    {65, 128, 1, 8192, 256, 512, 0, ANY, RULE_K_BELOW_4N, KERNEL_DECODE_RING},
+    {65, 128, 1, 4096, 513, 1024, 0, ANY, RULE_K_BELOW_4N, KERNEL_DECODE_RING},
+    // Against N >= 18432 (at least 144 column tiles, i.e. more than half the CUs busy without K slices): one launch
+    // of the hand-scheduled 128x128 tile, B copied with the non-temporal hint.  K = 2048 ... 8192 x N = 18432 ...
+    // 32768, M = 65 and 128: 3-50 % ahead of the split-K kernels (N = 28672, K = 4096, M = 128: 53.1 -> 48.6 us,
+    // 62.6 % of 8 TB/s); at N = 16384 mixed (0.84 ... 1.14), below it behind (0.79 ... 0.90).
+    {65, 128, 18432, ANY, 1024, ANY, 0, ANY, 0, KERNEL_MID128},
+    // --- everything else with N % 64 == 0 and K % 64 == 0: the split-K family, the tile by M; 128-wide tiles where
+    // N gives enough of them and is a multiple of 128 (they stream B better).
+    {1, 32, 1, ANY, 1, ANY, 0, ANY, 0, KERNEL_SPLIT_32x64},
+    {33, 64, 16384, ANY, 1, ANY, 0, ANY, 0, KERNEL_SPLIT_64x128},
+    {33, 64, 1, ANY, 1, ANY, 0, ANY, 0, KERNEL_SPLIT_64x64},
+    {65, 128, 16384, ANY, 1, ANY, 0, ANY, 0, KERNEL_SPLIT_128x128},
+    {65, 128, 1, ANY, 1, ANY, 0, ANY, 0, KERNEL_SPLIT_128x64},
+};
+constexpr int SMALL_M_RULE_COUNT = (int)(sizeof(SMALL_M_RULES) / sizeof(SMALL_M_RULES[0]));
+
+bool small_m_rule_covers(const SmallMRule &r, size_t M, size_t N, size_t K) {
+    const size_t b = N * K;
+    if (M < (size_t)r.m_lo || M > (size_t)r.m_hi || N < r.n_lo || N > r.n_hi || K < r.k_lo || K > r.k_hi || b < r.b_lo ||
+        b > r.b_hi)
+        return false;
+    if ((r.flags & RULE_K_BELOW_4N) && K >= 4 * N) return false;
+    if ((r.flags & RULE_K_NOT_16384S) && K % 16384 == 0) return false;
+    return true;
+}
+
+// shapes the kernel of a row can run at all (the row is skipped otherwise)
+bool small_m_kernel_supports(int kernel, size_t M, size_t N, size_t K) {
+    switch (kernel) {
+        case KERNEL_DECODE_RING: return decode_ring_supports(M, N, K);
+        case KERNEL_DECODE_BN16: return decode_supports(M, N, K);
+        case KERNEL_MID128: return N % 8 == 0 && K % 64 == 0 && K >= 64 * 5;
+        case KERNEL_SPLIT_64x128:
+        case KERNEL_SPLIT_128x128: return skinny_supports(M, N, K) && N % 128 == 0;
+        default: return skinny_supports(M, N, K);
+    }
+}
+
 }  // namespace
 
 bool skinny_supports(size_t M, size_t N, size_t K) {
@@ -330,49 +415,26 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     if (M == 0 || N == 0 || K == 0) return p;
     const size_t cus = (size_t)compute_units();
     const size_t slice_bytes = M * N * sizeof(float);  // fp32 partial sums of one K slice of the whole product
-    // a few rows: one streaming pass over B, no second launch; against a B of 96 MB or more the split-K kernel with
-    // B streamed past the caches is ahead from M = 6 (N = 14336: 8-16 %, N = 28672: 2-3 %; K = 4096)
-    const bool large_b = N * K >= ((size_t)48 << 20);
-    // M <= 128: the decode kernel with per-wave LDS rings, wherever it was measured ahead of the kernels below (K = 1024
-    // ... 28672 against N = 256 ... 28672, HBM-cold: 0-60 %, median 18 %).  Up to M = 8 that is everywhere except
-    // against a B of 96 MB or more with K < 8192 (ties) or K a multiple of 16384 (its 16 rows of B per workgroup then
-    // lie 32 KB apart: 20-28 % behind), and K < 2048 against N > 8192 (up to 4 % behind at M = 1).  Above M = 8 K slices
-    // across workgroups win from K = 5120 on unless N is small, and for N > 8192 or K >= 4 N.
-    const bool ring_small = !(large_b && (K < 8192 || K % 16384 == 0)) && !(K < 2048 && N > 8192);
-    const bool ring_mid = N <= 8192 && K < 4 * N && (K <= 4096 || (K <= 8192 && N <= 4096));
-    // M = 17 ... 64 (two or four row tiles of A per wave): while K is short, where one launch beats the split-K kernel
-    // and the launch that adds its slices.  Old library against new, K = 1024 ... 4096 against N = 272 ... 8192: ahead
-    // by 0-126 % (median 31 %, 180 shapes) for K <= 2048 up to N = 4096; beyond that mixed (M = 32: 15 % behind to 6 % ahead).
-    // (and up to K = 4096 for M <= 24 against N = 3072 ... 4096: 13-40 % ahead; at N <= 2048 M = 24 is 1-9 % behind)
-    const bool ring_tall = K < 4 * N && N <= (K < 1024 ? 8192u : 4096u) && (K <= 2048 || (M <= 24 && N >= 3072 && K <= 4096));
-    // K < 1024: up to M = 8 the streaming kernel is as fast or faster (one launch too); above, the same comparison
-    // (K = 256 ... 896 against N = 272 ... 8192) has the ring kernel ahead throughout
-    // M = 65 ... 128 (eight row tiles): K <= 1024 up to N = 4096, K <= 512 up to N = 8192 (15-100 % ahead)
-    const bool ring_tallest = K < 4 * N && K <= 1024 && N <= (K <= 512 ? 8192u : 4096u);
-    // (M <= 8 below K = 1024 only where the streaming kernel cannot run: N % 32 or K % 256 nonzero)
-    if (M <= 128 && decode_ring_supports(M, N, K) && K >= (M <= 8 && decode_supports(M, N, K) ? 1024u : 256u) &&
-        (M <= 8 ? ring_small : M <= 16 ? ring_mid : M <= 64 ? ring_tall : ring_tallest)) {
-        p.kernel = KERNEL_DECODE_RING;
-        p.splits = decode_ring_waves(M, N, K, cus);
-        return p;
-    }
-    if (M <= 8 && decode_supports(M, N, K) && !(M >= 6 && large_b && skinny_supports(M, N, K))) {
-        int bn = 16, waves = 1;
-        decode_plan(M, N, K, cus, &bn, &waves);
-        p.kernel = bn == 16 ? KERNEL_DECODE_BN16 : KERNEL_DECODE_BN32;
-        p.splits = waves;
-        return p;
-    }
-    if (skinny_supports(M, N, K)) {
-        const bool wide = M > 32 && N >= 16384 && N % 128 == 0;  // enough columns: 128-wide tiles stream B better
-        if (M <= 32)
-            p.kernel = KERNEL_SPLIT_32x64;
-        else if (M <= 64)
-            p.kernel = wide ? KERNEL_SPLIT_64x128 : KERNEL_SPLIT_64x64;
-        else
-            p.kernel = wide ? KERNEL_SPLIT_128x128 : KERNEL_SPLIT_128x64;
-        p.splits = choose_splits(N / (wide ? 128 : 64), cus, K, slice_bytes, limits.partial_bytes);
-        if (p.splits > 1) p.partial_bytes = (size_t)p.splits * slice_bytes;
+    // M <= 128: the first row of the table above that covers the shape and whose kernel can run it
+    for (const SmallMRule &r : SMALL_M_RULES) {
+        if (!small_m_rule_covers(r, M, N, K) || !small_m_kernel_supports(r.kernel, M, N, K)) continue;
+        p.kernel = r.kernel;
+        switch (r.kernel) {
+            case KERNEL_DECODE_RING: p.splits = decode_ring_waves(M, N, K, cus); break;
+            case KERNEL_DECODE_BN16: {  // the streaming kernel: 16 or 32 columns per workgroup
+                int bn = 16, waves = 1;
+                decode_plan(M, N, K, cus, &bn, &waves);
+                p.kernel = bn == 16 ? KERNEL_DECODE_BN16 : KERNEL_DECODE_BN32;
+                p.splits = waves;
+                break;
+            }
+            case KERNEL_MID128: p.splits = 1; break;
+            default: {  // the split-K family: K slices across workgroups, then the ordered reduction
+                const size_t bn = (r.kernel == KERNEL_SPLIT_64x128 || r.kernel == KERNEL_SPLIT_128x128) ? 128 : 64;
+                p.splits = choose_splits(N / bn, cus, K, slice_bytes, limits.partial_bytes);
+                if (p.splits > 1) p.partial_bytes = (size_t)p.splits * slice_bytes;
+            }
+        }
         return p;
     }
     // Pipelined tiles: M and N may end inside a tile (guarded edges; the model charges whole
@@ -737,6 +799,19 @@ extern "C" int hgemm_auto_plan_tail(size_t M, size_t N, size_t K, int *splits) {
     const Plan p = plan_for(M, N, K);
     if (splits) *splits = p.tail_splits;
     return p.tail_tiles;
+}
+// Row `index` of the table that decides the kernel for M <= 128 (first covering row whose kernel can run the shape
+// wins): bounds = {m_lo, m_hi, n_lo, n_hi, k_lo, k_hi, b_lo, b_hi}, inclusive, b = N * K; flags bit 0: only where
+// K < 4 N, bit 1: not where K is a multiple of 16384.  Returns the kernel id, or -1 past the end of the table.
+extern "C" int hgemm_small_m_rule(int index, size_t *bounds, int *flags) {
+    if (index < 0 || index >= SMALL_M_RULE_COUNT) return -1;
+    const SmallMRule &r = SMALL_M_RULES[index];
+    if (bounds) {
+        const size_t b[8] = {(size_t)r.m_lo, (size_t)r.m_hi, r.n_lo, r.n_hi, r.k_lo, r.k_hi, r.b_lo, r.b_hi};
+        for (int i = 0; i < 8; ++i) bounds[i] = b[i];
+    }
+    if (flags) *flags = r.flags;
+    return r.kernel;
 }
 // Kernel id of the smaller tile that takes over the last round (0: none).
 extern "C" int hgemm_auto_plan_tail_kernel(size_t M, size_t N, size_t K) { return plan_for(M, N, K).tail_kernel; }

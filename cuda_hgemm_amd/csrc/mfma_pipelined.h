@@ -133,10 +133,20 @@ struct MfmaOp<16> {
 // One MFMA slot that also starts a direct-to-LDS copy: M0 (the LDS destination) is set
 // before the MFMA, which doubles as the wait state the hardware wants between a write of
 // M0 and the copy that reads it, so the slot costs three instructions.
-template <int MI, int LDS_IMM>
+template <int MI, int LDS_IMM, bool NT = false>
 __device__ __forceinline__ void mfma_and_dma(half8 a, half8 b, typename MfmaOp<MI>::Acc &c, const void *sbase,
                                              uint32_t voff, uint32_t lds_base) {
-    if constexpr (MI == 16)
+    // NT: the copy carries the non-temporal hint (an operand that is read once and should not displace the other's
+    // panels from L2 and the Infinity Cache)
+    if constexpr (MI == 16 && NT)
+        asm volatile(
+            "s_add_u32 m0, %3, %6\n\t"
+            "v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\t"
+            "global_load_lds_dwordx4 %4, %5 nt"
+            : "+a"(c)
+            : "v"(a), "v"(b), "s"(lds_base), "v"(voff), "s"(sbase), "i"(LDS_IMM)
+            : "memory", "scc");
+    else if constexpr (MI == 16)
         asm volatile(
             "s_add_u32 m0, %3, %6\n\t"
             "v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\t"
@@ -152,6 +162,7 @@ __device__ __forceinline__ void mfma_and_dma(half8 a, half8 b, typename MfmaOp<M
             : "+a"(c)
             : "v"(a), "v"(b), "s"(lds_base), "v"(voff), "s"(sbase), "i"(LDS_IMM)
             : "memory", "scc");
+    static_assert(!NT || MI == 16, "the non-temporal copy is written for the 16x16x32 kernels");
 }
 
 // Ordered no-op that "modifies" an accumulator: later reads of it stay behind this point.
@@ -162,15 +173,24 @@ __device__ __forceinline__ void pin_accumulator(Acc &c) {
 
 // Direct-to-LDS copy: global address = scalar base + 32-bit per-lane byte offset, LDS
 // destination (wave-uniform, goes through M0) = lds_base + LDS_IMM.
-template <int LDS_IMM>
+template <int LDS_IMM, bool NT = false>
 __device__ __forceinline__ void dma_load16_sv(const void *sbase, uint32_t voff, uint32_t lds_base) {
-    asm volatile(
-        "s_add_u32 m0, %0, %3\n\t"
-        "s_nop 0\n\t"
-        "global_load_lds_dwordx4 %1, %2"
-        :
-        : "s"(lds_base), "v"(voff), "s"(sbase), "i"(LDS_IMM)
-        : "memory", "scc");
+    if constexpr (NT)
+        asm volatile(
+            "s_add_u32 m0, %0, %3\n\t"
+            "s_nop 0\n\t"
+            "global_load_lds_dwordx4 %1, %2 nt"
+            :
+            : "s"(lds_base), "v"(voff), "s"(sbase), "i"(LDS_IMM)
+            : "memory", "scc");
+    else
+        asm volatile(
+            "s_add_u32 m0, %0, %3\n\t"
+            "s_nop 0\n\t"
+            "global_load_lds_dwordx4 %1, %2"
+            :
+            : "s"(lds_base), "v"(voff), "s"(sbase), "i"(LDS_IMM)
+            : "memory", "scc");
 }
 
 // Accumulators -> fp16 -> C through LDS for either MFMA shape (operands swapped, so a lane
@@ -386,7 +406,10 @@ struct PipeFrame {
     }
 };
 
-template <class Cfg, bool SPLIT = false, bool EDGE = false>
+// STREAM_B: B's copies carry the non-temporal hint.  For one row of tiles against a B that outgrows the Infinity
+// Cache: every byte of B is read once, and as an ordinary read it pushes the A panel every workgroup shares out of
+// L2 and the Infinity Cache.
+template <class Cfg, bool SPLIT = false, bool EDGE = false, bool STREAM_B = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_pipelined_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
                            float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n,
@@ -419,7 +442,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         if constexpr (idx < A_DMA)
             dma_load16_sv<idx * Cfg::WAVES * 1024>(a_src, voff[idx], dst_a);
         else
-            dma_load16_sv<(idx - A_DMA) * Cfg::WAVES * 1024>(b_src, voff[idx], dst_b);
+            dma_load16_sv<(idx - A_DMA) * Cfg::WAVES * 1024, STREAM_B>(b_src, voff[idx], dst_b);
     };
 
     // Operand registers.  MFMAs run B-major (all A tiles against B tile 0, then B tile 1,
@@ -468,10 +491,11 @@ __global__ void __launch_bounds__(Cfg::THREADS)
         constexpr int imm = (d < A_DMA ? d : d - A_DMA) * Cfg::WAVES * 1024;
         const unsigned char *src = d < A_DMA ? a_src : b_src;
         const uint32_t dst = d < A_DMA ? dst_a : dst_b;
+        constexpr bool nt = STREAM_B && d >= A_DMA;
         if constexpr (j >= NSB)
-            mfma_and_dma<MI, imm>(b_last[fb][j - NSB], a_frag[fb][i], acc[i][j], src, voff[d], dst);
+            mfma_and_dma<MI, imm, nt>(b_last[fb][j - NSB], a_frag[fb][i], acc[i][j], src, voff[d], dst);
         else
-            mfma_and_dma<MI, imm>(b_frag[j], a_frag[fb][i], acc[i][j], src, voff[d], dst);
+            mfma_and_dma<MI, imm, nt>(b_frag[j], a_frag[fb][i], acc[i][j], src, voff[d], dst);
     };
 
     // ---- pipeline.  Chunk c of A lives in A-ring buffer c % SA, of B in B-ring buffer c % SB.
@@ -719,6 +743,19 @@ bool use_chained(PipeKernel which, size_t workgroups, size_t k_len) {
     return which == PipeKernel::Chained || chained_pays(Cfg::BM, Cfg::BN, workgroups, k_len);
 }
 
+// B copied with the non-temporal hint (the interleaved kernel's STREAM_B form): for one row of tiles against a
+// large B.  There every byte of B is read exactly once and A is one panel that every workgroup shares; B read the
+// ordinary way pushes that panel out of L2 and the Infinity Cache (128x128 tile, M = 128, N = 28672, K = 4096:
+// 52.8 -> 49.4 us).  From 48 MB of B on, the threshold the small-M split-K kernel uses for the same hint.  With two or
+// more rows of tiles B's panels are re-read by the rows below and the hint costs more than it returns, and on the
+// 256x128 and 256x256 tiles it is worth 2 % or less against their chained kernels (M = 256, N = 28672: 68.6 -> 67.3 us),
+// so only the 128x128 tile carries the second instantiation.
+template <class Cfg>
+constexpr bool stream_b_available() {
+    return Cfg::MI == 16 && Cfg::BM == 128 && Cfg::BN == 128 && Cfg::STAGES == 5;
+}
+inline bool stream_b_pays(int tiles_m, size_t N, size_t K) { return tiles_m == 1 && N * K >= ((size_t)24 << 20); }
+
 // Launches workgroup ids [first_block, first_block + blocks) of the tile grid; tail_tiles
 // as in the kernel.
 template <class Cfg, bool SPLIT, bool EDGE>
@@ -734,6 +771,10 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
             HGEMM_CHECK_HIP_ERROR(
                 hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_chained_kernel<Cfg, SPLIT, EDGE>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        if constexpr (stream_b_available<Cfg>() && !SPLIT)
+            HGEMM_CHECK_HIP_ERROR(
+                hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg, SPLIT, EDGE, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
         return true;
     }();
     (void)configured;
@@ -741,6 +782,15 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
     if (blocks < 0) blocks = tiles_m * tiles_n - first_block;
     HGEMM_CHECK(first_block >= 0 && blocks >= 1 && first_block + blocks <= tiles_m * tiles_n);
     HGEMM_CHECK(splits >= 1 && (SPLIT || splits == 1) && (size_t)blocks * (size_t)splits < ((size_t)1 << 31));
+    if constexpr (stream_b_available<Cfg>() && !SPLIT) {
+        if (which != PipeKernel::Chained && stream_b_pays(tiles_m, N, K)) {
+            hgemm_pipelined_kernel<Cfg, SPLIT, EDGE, true><<<dim3(blocks), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
+                reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
+                partial, (int)M, (int)N, (int)K, (int)K, tiles_m, tiles_n, first_block, tail_tiles, subdiv);
+            HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+            return;
+        }
+    }
     if constexpr (chained_available<Cfg>()) {
         if (use_chained<Cfg>(which, (size_t)blocks * (size_t)splits, K / (size_t)splits)) {
             hgemm_chained_kernel<Cfg, SPLIT, EDGE><<<dim3(blocks * splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(

@@ -135,6 +135,14 @@ int hgemm_auto_plan_tail_kernel(size_t M, size_t N, size_t K);
  * interleaved one (hgemm_mfma_pipelined_*) or a kernel of another family. */
 int hgemm_auto_plan_chained(size_t M, size_t N, size_t K);
 const char *hgemm_kernel_name(int kernel);
+/* The table behind hgemm_auto's choice for M <= 128 (decode-shaped products), row by row: the
+ * first row that covers a shape, and whose kernel can run it, decides.  bounds receives
+ * {m_lo, m_hi, n_lo, n_hi, k_lo, k_hi, b_lo, b_hi}, all inclusive, b = N * K (elements of B);
+ * flags bit 0: the row holds only where K < 4 N, bit 1: not where K is a multiple of 16384.
+ * Returns the row's kernel id (for hgemm_kernel_name; the streaming decode kernel's rows
+ * name its 16-column form and stand for both widths), or -1 past the last row.  No
+ * counterpart in the reference, which has no kernel for M < 256. */
+int hgemm_small_m_rule(int index, size_t *bounds, int *flags);
 
 /* ---- workspace of hgemm_auto / hgemm_skinny.  Plans that cut K into slices keep fp32
  * partial sums in device memory, and large shapes with N % 8 != 0 or K % 64 != 0 run on

@@ -112,12 +112,68 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
                 assert ("LDS ring per K slice" in p["kernel"]) == (n == 4096), (m, n, p)
             elif m == 16 and n == 4096:                     # up to M = 16 the decode kernel with per-wave LDS rings
                 assert "LDS ring per K slice" in p["kernel"] and p["splits"] == 4, (m, n, p)
+            elif m == 128 and n == 28672:                   # one tile row against 224 column tiles: one launch
+                assert p["kernel"].startswith("pipelined 128x128x64") and p["splits"] == 1, (m, n, p)
             else:
                 assert p["kernel"].startswith("split-K"), (m, n, p)
             assert 4096 % (p["splits"] * 64) == 0
     assert plan(100, 100, 100)["kernel"].startswith("guarded 128x128x32")      # no tile divides it
     assert plan(1000, 4000, 4096)["kernel"].startswith("pipelined")            # ragged M, N: guarded edges
     assert plan(4095, 4095, 4095)["kernel"].startswith("zero-padded")          # large and unaligned
+
+
+def test_small_m_rule_table(hgemm_lib):
+    """The table that decides the kernel for M <= 128 is data the library hands out: its rows are well-formed boxes,
+    every M in 1 ... 128 ends in a catch-all row of the split-K family, and hgemm_auto's plan is the first covering
+    row whose kernel can run the shape -- looked up here independently over a grid of shapes."""
+    rules = hgemm_lib.small_m_rules()
+    assert 15 <= len(rules) <= 40, len(rules)
+    for r in rules:
+        assert 1 <= r["m_lo"] <= r["m_hi"] <= 128 and r["n_lo"] <= r["n_hi"] and r["k_lo"] <= r["k_hi"], r
+        assert r["b_lo"] <= r["b_hi"] and r["kernel"] != "none", r
+    for m in range(1, 129):
+        last = [r for r in rules if r["m_lo"] <= m <= r["m_hi"]][-1]
+        assert last["kernel"].startswith("split-K") and last["n_lo"] <= 64 and last["k_lo"] <= 64, (m, last)
+        assert last["n_hi"] > 1 << 40 and last["k_hi"] > 1 << 40 and not last["k_below_4n"], (m, last)
+
+    def can_run(kernel, M, N, K):
+        if "LDS ring per K slice" in kernel:
+            return N % 16 == 0 and K % 128 == 0
+        if kernel.startswith("streaming decode"):
+            return M <= 32 and N % 32 == 0 and K % 256 == 0
+        if kernel.startswith("pipelined 128x128"):
+            return N % 8 == 0 and K % 64 == 0 and K >= 320
+        if kernel.startswith("split-K"):
+            wide = kernel.split()[1].split("x")[1] == "128"       # "split-K <BM>x<BN>x64, ...": 128-column tiles
+            return N % 64 == 0 and K % 64 == 0 and (N % 128 == 0 or not wide)
+        raise AssertionError(kernel)
+
+    def lookup(M, N, K):
+        for r in rules:
+            if not (r["m_lo"] <= M <= r["m_hi"] and r["n_lo"] <= N <= r["n_hi"] and r["k_lo"] <= K <= r["k_hi"]
+                    and r["b_lo"] <= N * K <= r["b_hi"]):
+                continue
+            if (r["k_below_4n"] and K >= 4 * N) or (r["k_not_multiple_of_16384"] and K % 16384 == 0):
+                continue
+            if can_run(r["kernel"], M, N, K):
+                return r["kernel"]
+        return None
+
+    family = lambda name: name.split(",")[0].replace("32 columns", "16 columns")   # the streaming kernel's two widths
+    checked = 0
+    for M in (1, 5, 6, 8, 9, 16, 17, 24, 25, 64, 65, 100, 128):
+        for N in (16, 48, 64, 272, 2048, 3072, 4096, 4112, 8192, 8208, 14336, 16384, 18432, 20488, 28672, 57344):
+            for K in (64, 256, 384, 512, 1024, 1152, 2048, 2304, 4096, 4160, 8192, 12288, 16384, 32768):
+                expect = lookup(M, N, K)
+                if expect is None:
+                    continue
+                got = hgemm_lib.auto_plan(M, N, K)["kernel"]
+                assert family(got) == family(expect), (M, N, K, got, expect)
+                checked += 1
+    assert checked > 2000, checked
+    # the headline decode shapes, by row
+    assert lookup(1, 4096, 4096).endswith("one LDS ring per K slice") and lookup(128, 4096, 4096).startswith("split-K 128x64")
+    assert lookup(1, 28672, 4096).startswith("streaming decode, 16") and lookup(128, 28672, 4096).startswith("pipelined 128x128")
 
 
 def test_auto_plan_invariants_over_many_shapes(hgemm_lib):
