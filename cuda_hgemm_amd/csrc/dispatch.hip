@@ -163,6 +163,8 @@ using Mid128 = PipeConfig<128, 128, 64, 2, 2, 5, 16>;
 // a workgroup's K loop is shorter than its epilogue and C outgrows the Infinity Cache: 16384^2 x 256 201 -> 170 us.
 using Mid128S2 = PipeConfig<128, 128, 64, 2, 2, 2, 16>;
 using Small64 = PipeConfig<64, 64, 64, 1, 1, 3, 16>;
+// one row of tiles for M <= 64: four waves side by side, 64x32 each
+using Row64x128 = PipeConfig<64, 128, 64, 1, 4, 5, 16>;
 using Tile192 = PipeConfig<192, 192, 64, 2, 2, 3, 16>;
 using Rect256x128 = PipeConfig<256, 128, 64, 2, 2, 3, 16>;
 // 64x64x64 on four waves (one 32x32 MFMA tile each) with the ladder's kernel: a small tile whose chunk takes a quarter
@@ -367,8 +369,13 @@ constexpr SmallMRule SMALL_M_RULES[] = {
     // Against N >= 18432 (at least 144 column tiles, i.e. more than half the CUs busy without K slices): one launch
     // of the hand-scheduled 128x128 tile, B copied with the non-temporal hint.  K = 2048 ... 8192 x N = 18432 ...
     // 32768, M = 65 and 128: 3-50 % ahead of the split-K kernels (N = 28672, K = 4096, M = 128: 53.1 -> 48.6 us,
-    // 62.6 % of 8 TB/s); at N = 16384 mixed (0.84 ... 1.14), below it behind (0.79 ... 0.90).
-    {65, 128, 18432, ANY, 1024, ANY, 0, ANY, 0, KERNEL_MID128},
+    // 62.6 % of 8 TB/s), K = 384 ... 768 x N = 28672, 57344: 1.11 ... 1.24x; at N = 16384 mixed (0.84 ... 1.14), below
+    // it behind (0.76 ... 0.90).  From K = 320, the shortest K its five-stage ring takes.
+    {65, 128, 18432, ANY, 320, ANY, 0, ANY, 0, KERNEL_MID128},
+    // M = 33 ... 64 there: the same kernel on a 64x128 tile, four waves side by side.  K = 384 ... 8192 x N = 18432 ...
+    // 57344: 1-4 % ahead of the split-K 64x128 kernel where that ran unsliced (N = 28672, K = 4096, M = 64: 43.3 ->
+    // 42.4 us, 70 % of 8 TB/s), 1.35x where it ran in two slices (N = 18432, 20480).
+    {33, 64, 18432, ANY, 320, ANY, 0, ANY, 0, KERNEL_ROW64x128},
     // --- everything else with N % 64 == 0 and K % 64 == 0: the split-K family, the tile by M; 128-wide tiles where
     // N gives enough of them and is a multiple of 128 (they stream B better).
     {1, 32, 1, ANY, 1, ANY, 0, ANY, 0, KERNEL_SPLIT_32x64},
@@ -394,7 +401,8 @@ bool small_m_kernel_supports(int kernel, size_t M, size_t N, size_t K) {
     switch (kernel) {
         case KERNEL_DECODE_RING: return decode_ring_supports(M, N, K);
         case KERNEL_DECODE_BN16: return decode_supports(M, N, K);
-        case KERNEL_MID128: return N % 8 == 0 && K % 64 == 0 && K >= 64 * 5;
+        case KERNEL_MID128:
+        case KERNEL_ROW64x128: return N % 8 == 0 && K % 64 == 0 && K >= 64 * 5;
         case KERNEL_SPLIT_64x128:
         case KERNEL_SPLIT_128x128: return skinny_supports(M, N, K) && N % 128 == 0;
         default: return skinny_supports(M, N, K);
@@ -428,7 +436,8 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
                 p.splits = waves;
                 break;
             }
-            case KERNEL_MID128: p.splits = 1; break;
+            case KERNEL_MID128:
+            case KERNEL_ROW64x128: p.splits = 1; break;
             default: {  // the split-K family: K slices across workgroups, then the ordered reduction
                 const size_t bn = (r.kernel == KERNEL_SPLIT_64x128 || r.kernel == KERNEL_SPLIT_128x128) ? 128 : 64;
                 p.splits = choose_splits(N / bn, cus, K, slice_bytes, limits.partial_bytes);
@@ -606,6 +615,7 @@ void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, 
         case KERNEL_R256x128: launch_pipelined_plan<Rect256x128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128_S2: launch_pipelined<Mid128S2>(A, B, C, M, N, K, "hgemm_auto"); break;
+        case KERNEL_ROW64x128: launch_pipelined<Row64x128>(A, B, C, M, N, K, "hgemm_auto"); break;
         case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_SMALL64_W4: {
             const size_t chunks = K / 64 / (size_t)(p.splits > 1 ? p.splits : 1);
@@ -835,6 +845,7 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
         case KERNEL_BIG256: return "pipelined 256x256x64, 4 waves, LDS ring 3 (A) + 2 (B)";
         case KERNEL_MID128: return "pipelined 128x128x64, 4 waves, 5-stage ring";
         case KERNEL_MID128_S2: return "pipelined 128x128x64, 4 waves, 2-stage ring";
+        case KERNEL_ROW64x128: return "pipelined 64x128x64, 4 waves, 5-stage ring";
         case KERNEL_SMALL64: return "pipelined 64x64x64, 1 wave, 3-stage ring";
         case KERNEL_SMALL64_W4: return "tiled 64x64x64, 4 waves of 32x32, look-ahead ring";
         case KERNEL_T192: return "pipelined 192x192x64, 4 waves, 3-stage ring";

@@ -749,10 +749,10 @@ bool use_chained(PipeKernel which, size_t workgroups, size_t k_len) {
 // 52.8 -> 49.4 us).  From 48 MB of B on, the threshold the small-M split-K kernel uses for the same hint.  With two or
 // more rows of tiles B's panels are re-read by the rows below and the hint costs more than it returns, and on the
 // 256x128 and 256x256 tiles it is worth 2 % or less against their chained kernels (M = 256, N = 28672: 68.6 -> 67.3 us),
-// so only the 128x128 tile carries the second instantiation.
+// so only the tiles that run one row against many columns (128x128, 64x128; five stages) carry the second instantiation.
 template <class Cfg>
 constexpr bool stream_b_available() {
-    return Cfg::MI == 16 && Cfg::BM == 128 && Cfg::BN == 128 && Cfg::STAGES == 5;
+    return Cfg::MI == 16 && Cfg::BN == 128 && (Cfg::BM == 128 || Cfg::BM == 64) && Cfg::STAGES == 5;
 }
 inline bool stream_b_pays(int tiles_m, size_t N, size_t K) { return tiles_m == 1 && N * K >= ((size_t)24 << 20); }
 

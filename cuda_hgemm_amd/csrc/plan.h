@@ -25,6 +25,7 @@ enum KernelId {
     KERNEL_MID128_S2,   // pipelined 128x128x64, 4 waves, 2-stage ring: two workgroups per CU, for K of at most four chunks
     KERNEL_DECODE_RING, // decode kernel for M <= 128 whose waves stage operands through LDS rings of their own; `splits` waves over K
     KERNEL_PADDED,      // operands copied zero-padded to N % 8 == 0, K % 64 == 0, then the plan for that shape
+    KERNEL_ROW64x128,   // pipelined 64x128x64, 4 waves side by side, 5-stage ring: one row of tiles for M <= 64 against many columns
 };
 
 struct Plan {

@@ -50,7 +50,7 @@ def _row(lib, kind, m, n, k, ms, vms, extra=None):
 
 
 def run(lib, vendor, warmup=10, steps=100):
-    """Every size with `warmup` untimed and `steps` timed launches, the vendor GEMM first."""
+    """Every size with `warmup` untimed and `steps` timed launches per pass, two passes each, the vendor GEMM first."""
     import numpy as np
     from . import hipmem
     dev_array = hipmem.DeviceArray
@@ -61,8 +61,12 @@ def run(lib, vendor, warmup=10, steps=100):
     def one(kind, m, n, k, dist_a, dist_b):
         A, B = dev_array.from_host(_draw(rng, m, k, dist_a)), dev_array.from_host(_draw(rng, n, k, dist_b))
         C = dev_array((m, n))
+        # the vendor GEMM first, as the reference's driver runs cuBLAS first; both twice, alternating, the better pass
+        # of each kept (the part is power-managed: whoever runs second in a pair meets a different clock)
         vms = _time(hipmem, lib, vfn, [A], [B], [C], m, n, k, warmup, steps)
         ms = _time(hipmem, lib, auto, [A], [B], [C], m, n, k, warmup, steps)
+        vms = min(vms, _time(hipmem, lib, vfn, [A], [B], [C], m, n, k, warmup, steps))
+        ms = min(ms, _time(hipmem, lib, auto, [A], [B], [C], m, n, k, warmup, steps))
         rows.append(_row(lib, kind, m, n, k, ms, vms, {"vendor_pick": vendor.candidates(m, n, k)}))
         for buf in (A, B, C):
             buf.free()
@@ -82,8 +86,10 @@ def run(lib, vendor, warmup=10, steps=100):
             As = [dev_array.from_host(np.roll(a_base, i, axis=1)) for i in range(copies)]
             Cs = [dev_array((m, n)) for _ in range(copies)]
             warm_ms = _time(hipmem, lib, auto, As[:1], Bs[:1], Cs[:1], m, n, k, warmup, steps)
-            cold_ms = _time(hipmem, lib, auto, As, Bs, Cs, m, n, k, warmup, steps)
             vcold_ms = _time(hipmem, lib, vfn, As, Bs, Cs, m, n, k, warmup, steps)
+            cold_ms = _time(hipmem, lib, auto, As, Bs, Cs, m, n, k, warmup, steps)
+            vcold_ms = min(vcold_ms, _time(hipmem, lib, vfn, As, Bs, Cs, m, n, k, warmup, steps))
+            cold_ms = min(cold_ms, _time(hipmem, lib, auto, As, Bs, Cs, m, n, k, warmup, steps))
             rows.append(_row(lib, "decode", m, n, k, cold_ms, vcold_ms,
                              {"cache_warm_ms": warm_ms, "cache_warm_gbps": lib.bytes(m, n, k) / (warm_ms * 1e-3) * 1e-9,
                               "operand_sets": copies, "vendor_pick": vendor.candidates(m, n, k)}))

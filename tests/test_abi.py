@@ -112,8 +112,8 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
                 assert ("LDS ring per K slice" in p["kernel"]) == (n == 4096), (m, n, p)
             elif m == 16 and n == 4096:                     # up to M = 16 the decode kernel with per-wave LDS rings
                 assert "LDS ring per K slice" in p["kernel"] and p["splits"] == 4, (m, n, p)
-            elif m == 128 and n == 28672:                   # one tile row against 224 column tiles: one launch
-                assert p["kernel"].startswith("pipelined 128x128x64") and p["splits"] == 1, (m, n, p)
+            elif m >= 64 and n == 28672:                    # one tile row against 224 column tiles: one launch
+                assert p["kernel"].startswith("pipelined %dx128x64" % m) and p["splits"] == 1, (m, n, p)
             else:
                 assert p["kernel"].startswith("split-K"), (m, n, p)
             assert 4096 % (p["splits"] * 64) == 0
@@ -141,7 +141,7 @@ def test_small_m_rule_table(hgemm_lib):
             return N % 16 == 0 and K % 128 == 0
         if kernel.startswith("streaming decode"):
             return M <= 32 and N % 32 == 0 and K % 256 == 0
-        if kernel.startswith("pipelined 128x128"):
+        if kernel.startswith(("pipelined 128x128", "pipelined 64x128")):
             return N % 8 == 0 and K % 64 == 0 and K >= 320
         if kernel.startswith("split-K"):
             wide = kernel.split()[1].split("x")[1] == "128"       # "split-K <BM>x<BN>x64, ...": 128-column tiles
@@ -161,7 +161,7 @@ def test_small_m_rule_table(hgemm_lib):
 
     family = lambda name: name.split(",")[0].replace("32 columns", "16 columns")   # the streaming kernel's two widths
     checked = 0
-    for M in (1, 5, 6, 8, 9, 16, 17, 24, 25, 64, 65, 100, 128):
+    for M in (1, 5, 6, 8, 9, 16, 17, 24, 25, 32, 33, 64, 65, 100, 128):
         for N in (16, 48, 64, 272, 2048, 3072, 4096, 4112, 8192, 8208, 14336, 16384, 18432, 20488, 28672, 57344):
             for K in (64, 256, 384, 512, 1024, 1152, 2048, 2304, 4096, 4160, 8192, 12288, 16384, 32768):
                 expect = lookup(M, N, K)
@@ -174,6 +174,7 @@ def test_small_m_rule_table(hgemm_lib):
     # the headline decode shapes, by row
     assert lookup(1, 4096, 4096).endswith("one LDS ring per K slice") and lookup(128, 4096, 4096).startswith("split-K 128x64")
     assert lookup(1, 28672, 4096).startswith("streaming decode, 16") and lookup(128, 28672, 4096).startswith("pipelined 128x128")
+    assert lookup(64, 28672, 4096).startswith("pipelined 64x128") and lookup(16, 28672, 4096).startswith("split-K 32x64")
 
 
 def test_auto_plan_invariants_over_many_shapes(hgemm_lib):
