@@ -341,20 +341,30 @@ constexpr SmallMRule SMALL_M_RULES[] = {
     // --- M = 1 ... 8.  Below K = 1024 the streaming kernel (as fast or faster, M = 1 by 6-26 %) where it can run,
     // i.e. N % 32 == 0 and K % 256 == 0; else the ring kernel (2.0x median over what ran such shapes before).
     {1, 8, 1, 8192, 256, 1023, 0, ANY, 0, KERNEL_DECODE_BN16},
-    // The ring kernel: 0-60 % ahead (median 18 %) except against a B of 96 MB or more with K < 8192 (ties at M <= 8,
-    // the split-K kernel streams B past the caches there) and except K < 2048 against N > 8192 (up to 4 % behind).
+    // The ring kernel: 0-60 % ahead (median 18 %); not for K < 2048 against N > 8192 (up to 4 % behind at M = 1).  Its
+    // copies of B carry the non-temporal hint from 48 MB of B on, and with the hint it is also ahead against a B of
+    // 96 MB or more, where the streaming and split-K kernels used to tie with it: K = 1024 ... 12288 x N = 10240 ...
+    // 57344, M = 1: 0.97 ... 1.18x (N = 28672, K = 4096: 39.2 -> 35.9 us, 82 % of 8 TB/s; N = 57344: 87 %), M = 8:
+    // 0.95 ... 1.31x from K = 2048 (ties at K = 1024).
     {1, 8, 1, 8192, 256, 2047, 0, ANY, 0, KERNEL_DECODE_RING},
     {1, 8, 1, ANY, 2048, 8191, 0, LARGE_B - 1, 0, KERNEL_DECODE_RING},
     {1, 8, 1, ANY, 8192, ANY, 0, LARGE_B - 1, 0, KERNEL_DECODE_RING},
     {1, 8, 1, ANY, 8192, ANY, LARGE_B, ANY, RULE_K_NOT_16384S, KERNEL_DECODE_RING},
-    // M = 6 ... 8 against a B of 96 MB or more: the split-K kernel (N = 14336: 8-16 % ahead of the streaming kernel,
-    // N = 28672: 2-3 %); below M = 6 and for smaller B the streaming kernel stays ahead.
+    {1, 5, 1, ANY, 1024, 8191, LARGE_B, ANY, 0, KERNEL_DECODE_RING},
+    {6, 8, 1, ANY, 2048, 8191, LARGE_B, ANY, 0, KERNEL_DECODE_RING},
+    // M = 6 ... 8 against a B of 96 MB or more with K < 2048: the split-K kernel (2-16 % ahead of the streaming
+    // kernel); below M = 6 and for smaller B the streaming kernel stays ahead.
     {6, 8, 1, ANY, 1, ANY, LARGE_B, ANY, 0, KERNEL_SPLIT_32x64},
     {1, 8, 1, ANY, 1, ANY, 0, ANY, 0, KERNEL_DECODE_BN16},
     // --- M = 9 ... 16: the ring kernel up to N = 8192 while K <= 4096 (K <= 8192 up to N = 4096); beyond, K slices
-    // across workgroups are up to 29 % ahead.
+    // across workgroups are up to 29 % ahead -- except, with the non-temporal copies, against a B of 48 MB or more at
+    // K = 2048, 4096 and 8192, where every wave walks 1024 of K (M = 12: 1.05 ... 1.29x, M = 16: 0.97 ... 1.23x over
+    // N = 10240 ... 57344); at K = 1024, 3072, 6144 and 12288 the split-K kernel stays ahead (0.84 ... 1.06x).
     {9, 16, 1, 8192, 256, 4096, 0, ANY, RULE_K_BELOW_4N, KERNEL_DECODE_RING},
     {9, 16, 1, 4096, 4097, 8192, 0, ANY, RULE_K_BELOW_4N, KERNEL_DECODE_RING},
+    {9, 16, 8193, ANY, 2048, 2048, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RING},
+    {9, 16, 8193, ANY, 4096, 4096, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RING},
+    {9, 16, 8193, ANY, 8192, 8192, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RING},
     // --- M = 17 ... 64 (two or four row tiles of A per wave): the ring kernel while K is short, where one launch beats
     // the split-K kernel plus the launch that adds its slices: K < 1024 up to N = 8192 (median 1.65x), K <= 2048 up
     // to N = 4096 (median 1.31x); and up to K = 4096 for M <= 24 against N = 3072 ... 4096 (median 1.21x; at

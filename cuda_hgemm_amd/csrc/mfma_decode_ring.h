@@ -44,7 +44,9 @@ struct RingConfig {
                   "wait count range; the ring takes the wave's partial sums");
 };
 
-template <int TM, int STAGES>
+// STREAM_B: B's copies carry the non-temporal hint (every byte of B is read once; the launcher sets it from 48 MB of B on,
+// the threshold the split-K kernel uses for the same hint).
+template <int TM, int STAGES, bool STREAM_B = false>
 __global__ void __launch_bounds__(RING_MAX_WAVES * 64)
     hgemm_decode_ring_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C, int M,
                              int N, int K, int k_per_wave) {
@@ -74,8 +76,13 @@ __global__ void __launch_bounds__(RING_MAX_WAVES * 64)
         const uint32_t base = ring_addr + slot * RING_CHUNK_BYTES;
 #pragma unroll
         for (int h = 0; h < 2 * TM; ++h) dma_load16(a_src[h] + kt * 64, base + h * 1024);
-        dma_load16(b_src[0] + kt * 64, base + A_BYTES);
-        dma_load16(b_src[1] + kt * 64, base + A_BYTES + 1024);
+        if constexpr (STREAM_B) {
+            dma_load16_streaming(b_src[0] + kt * 64, base + A_BYTES);
+            dma_load16_streaming(b_src[1] + kt * 64, base + A_BYTES + 1024);
+        } else {
+            dma_load16(b_src[0] + kt * 64, base + A_BYTES);
+            dma_load16(b_src[1] + kt * 64, base + A_BYTES + 1024);
+        }
     };
 
     // ---- operands of the two 32-wide steps of a chunk: lane l holds row l % 16 (of each 16-row tile), pieces l / 16
@@ -164,15 +171,18 @@ void launch_decode_ring_tile(const void *A, const void *B, void *C, size_t M, si
     using Cfg = RingConfig<TM, STAGES>;
     HGEMM_CHECK((size_t)waves * Cfg::RING_BYTES <= 160 * 1024);
     static bool configured = [] {
-        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_decode_ring_kernel<TM, STAGES>),
+        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_decode_ring_kernel<TM, STAGES, false>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_decode_ring_kernel<TM, STAGES, true>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         return true;
     }();
     (void)configured;
-    hgemm_decode_ring_kernel<TM, STAGES><<<dim3((unsigned)(N / 16)), dim3(waves * 64), (size_t)waves * Cfg::RING_BYTES,
-                                           nullptr>>>(reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B),
-                                                      reinterpret_cast<half_t *>(C), (int)M, (int)N, (int)K,
-                                                      (int)(K / (size_t)waves));
+    auto kernel = N * K >= ((size_t)24 << 20) ? &hgemm_decode_ring_kernel<TM, STAGES, true>
+                                              : &hgemm_decode_ring_kernel<TM, STAGES, false>;
+    kernel<<<dim3((unsigned)(N / 16)), dim3(waves * 64), (size_t)waves * Cfg::RING_BYTES, nullptr>>>(
+        reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), (int)M,
+        (int)N, (int)K, (int)(K / (size_t)waves));
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 

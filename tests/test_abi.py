@@ -107,16 +107,15 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
     for m in (1, 8, 16, 64, 128):
         for n in (4096, 28672):
             p = plan(m, n, 4096)
-            if m <= 8 and not (m >= 6 and n == 28672):     # from M = 6 a B of 96 MB or more goes to the split-K kernel
-                assert p["kernel"].startswith("streaming decode"), (m, n, p)
-                assert ("LDS ring per K slice" in p["kernel"]) == (n == 4096), (m, n, p)
-            elif m == 16 and n == 4096:                     # up to M = 16 the decode kernel with per-wave LDS rings
+            if m <= 16:      # the decode kernel with per-wave LDS rings (B copied non-temporally at N = 28672)
                 assert "LDS ring per K slice" in p["kernel"] and p["splits"] == 4, (m, n, p)
-            elif m >= 64 and n == 28672:                    # one tile row against 224 column tiles: one launch
+            elif n == 28672:                                # one tile row against 224 column tiles: one launch
                 assert p["kernel"].startswith("pipelined %dx128x64" % m) and p["splits"] == 1, (m, n, p)
             else:
                 assert p["kernel"].startswith("split-K"), (m, n, p)
             assert 4096 % (p["splits"] * 64) == 0
+    assert plan(4, 28672, 512)["kernel"].startswith("streaming decode, 16 columns per workgroup, one wave per K slice")
+    assert plan(7, 57344, 1024)["kernel"].startswith("split-K 32x64")
     assert plan(100, 100, 100)["kernel"].startswith("guarded 128x128x32")      # no tile divides it
     assert plan(1000, 4000, 4096)["kernel"].startswith("pipelined")            # ragged M, N: guarded edges
     assert plan(4095, 4095, 4095)["kernel"].startswith("zero-padded")          # large and unaligned
@@ -173,8 +172,9 @@ def test_small_m_rule_table(hgemm_lib):
     assert checked > 2000, checked
     # the headline decode shapes, by row
     assert lookup(1, 4096, 4096).endswith("one LDS ring per K slice") and lookup(128, 4096, 4096).startswith("split-K 128x64")
-    assert lookup(1, 28672, 4096).startswith("streaming decode, 16") and lookup(128, 28672, 4096).startswith("pipelined 128x128")
-    assert lookup(64, 28672, 4096).startswith("pipelined 64x128") and lookup(16, 28672, 4096).startswith("split-K 32x64")
+    assert lookup(1, 28672, 4096).endswith("one LDS ring per K slice") and lookup(128, 28672, 4096).startswith("pipelined 128x128")
+    assert lookup(64, 28672, 4096).startswith("pipelined 64x128") and lookup(16, 28672, 4096).endswith("one LDS ring per K slice")
+    assert lookup(16, 28672, 3072).startswith("split-K 32x64") and lookup(2, 28672, 512).startswith("streaming decode, 16")
 
 
 def test_auto_plan_invariants_over_many_shapes(hgemm_lib):

@@ -376,7 +376,10 @@ def test_streaming_decode_kernel(oracle, hgemm_lib, gpu, shape):
                                    (5, 8192, 8192), (7, 4112, 16384 - 128), (17, 4096, 2048), (32, 4096, 1024),
                                    (24, 1040, 1280), (33, 4096, 2048), (64, 4096, 1024), (48, 2064, 1152), (40, 272, 1024),
                                    (16, 4096, 256), (64, 8192, 896), (33, 272, 384), (9, 1040, 640),
-                                   (65, 4096, 1024), (128, 8192, 512), (100, 272, 384), (128, 4096, 256), (24, 4096, 4096), (5, 1040, 384), (8, 4096, 640)])
+                                   (65, 4096, 1024), (128, 8192, 512), (100, 272, 384), (128, 4096, 256), (24, 4096, 4096), (5, 1040, 384), (8, 4096, 640),
+                                   # B of 48 MB or more: the copies of B carry the non-temporal hint
+                                   (1, 28672, 4096), (8, 28672, 4096), (16, 28672, 4096), (5, 14336, 4096), (12, 16384, 8192),
+                                   (3, 57344, 1024), (7, 28672, 2048), (8, 20480, 2816), (6, 14336, 4096), (16, 8192, 4096)])
 def test_decode_kernel_with_lds_rings(oracle, hgemm_lib, gpu, shape):
     """M <= 128 through per-wave LDS rings (one, two, four or eight 16-row tiles of A per wave): one, two, four and eight K slices per workgroup, slices of one chunk and of
     many (127 when only two waves divide K), slices shorter than the ring, N of one to 896 column tiles, rows of A
@@ -393,9 +396,10 @@ def test_decode_kernel_with_lds_rings(oracle, hgemm_lib, gpu, shape):
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
-@pytest.mark.parametrize("shape", [(7, 28672, 2048), (8, 20480, 2816), (6, 14336, 4096), (100, 14336, 4096)])
+@pytest.mark.parametrize("shape", [(7, 57344, 1024), (8, 65536, 1536), (12, 28672, 3072), (100, 14336, 4096)])
 def test_small_m_against_a_large_b(oracle, hgemm_lib, gpu, shape):
-    """B of 96 MB or more: from M = 6 the split-K kernel runs, with B copied past the caches (non-temporal hint)."""
+    """B of 96 MB or more where the split-K kernel runs, with B copied past the caches (non-temporal hint): M = 6 ... 8
+    while K < 2048, M = 9 ... 16 at the K where it is ahead of the ring kernel, M = 65 ... 128 below 144 column tiles."""
     M, N, K = shape
     assert hgemm_lib.auto_plan(M, N, K)["kernel"].startswith("split-K")
     A = oracle.fill((M, K), 33, 1, oracle.NORMAL, 0.0, 1.0)
