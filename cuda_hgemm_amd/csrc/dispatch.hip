@@ -386,6 +386,10 @@ constexpr SmallMRule SMALL_M_RULES[] = {
     // 57344: 1-4 % ahead of the split-K 64x128 kernel where that ran unsliced (N = 28672, K = 4096, M = 64: 43.3 ->
     // 42.4 us, 70 % of 8 TB/s), 1.35x where it ran in two slices (N = 18432, 20480).
     {33, 64, 18432, ANY, 320, ANY, 0, ANY, 0, KERNEL_ROW64x128},
+    // M = 17 ... 32 take that tile too once K is long (half its rows are idle, which an HBM-bound kernel can afford):
+    // K = 4096, 8192 x N = 18432 ... 57344: 0.97 ... 1.27x over the split-K 32x64 kernel; at K <= 2048 that kernel stays
+    // ahead against N >= 28672 (0.92 ... 0.98x).
+    {17, 32, 18432, ANY, 4096, ANY, 0, ANY, 0, KERNEL_ROW64x128},
     // --- everything else with N % 64 == 0 and K % 64 == 0: the split-K family, the tile by M; 128-wide tiles where
     // N gives enough of them and is a multiple of 128 (they stream B better).
     {1, 32, 1, ANY, 1, ANY, 0, ANY, 0, KERNEL_SPLIT_32x64},

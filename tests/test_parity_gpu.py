@@ -414,14 +414,14 @@ def test_small_m_against_a_large_b(oracle, hgemm_lib, gpu, shape):
 @pytest.mark.parametrize("shape", [(128, 28672, 4096), (100, 18440, 1024), (65, 20480, 2048), (128, 18432, 1088),
                                    (97, 24584, 1024), (128, 28672, 320 + 704),
                                    (64, 28672, 4096), (33, 18440, 1024), (50, 20480, 2048), (64, 24584, 1088), (64, 28672, 320),
-                                   (128, 28672, 384)])
+                                   (128, 28672, 384), (17, 28672, 4096), (32, 18432, 8192)])
 def test_one_tile_row_against_many_column_tiles(oracle, hgemm_lib, gpu, shape):
     """M = 33 ... 128 against N >= 18432: one launch of the pipelined kernel on a 128x128 tile (a 64x128 tile up to
     M = 64) whose copies of B carry the non-temporal hint (from 48 MB of B on; the smaller cases run the same rule
     without the hint), rows of the tile beyond M and a last column tile that ends inside the tile included."""
     M, N, K = shape
     plan = hgemm_lib.auto_plan(M, N, K)
-    tile = "128x128x64" if M > 64 else "64x128x64"
+    tile = "128x128x64" if M > 64 else "64x128x64"      # M = 17 ... 32 join the 64x128 tile from K = 4096
     assert plan["kernel"].startswith(f"pipelined {tile}, 4 waves, 5-stage") and plan["splits"] == 1, plan
     A = oracle.fill((M, K), 41, 1, oracle.NORMAL, 0.0, 1.0)
     B = oracle.fill((N, K), 41, 2, oracle.NORMAL, 0.0, 0.02)
