@@ -2,6 +2,7 @@
 #include "../../include/hgemm.h"
 #include "mfma_decode.h"
 #include "mfma_decode_ring.h"
+#include "mfma_decode_resident.h"
 #include "mfma_pipelined.h"
 #include "mfma_ragged.h"
 #include "mfma_skinny.h"
@@ -129,7 +130,7 @@ void launch_splitk(const void *A, const void *B, void *C, size_t M, size_t N, si
     }();
     (void)configured;
     HGEMM_CHECK(N % Cfg::BN == 0);
-    HGEMM_CHECK(splits >= 1 && K % ((size_t)splits * Cfg::BK) == 0);
+    HGEMM_CHECK(splits >= 1 && K % (size_t)Cfg::BK == 0 && K / (size_t)Cfg::BK >= (size_t)splits);
     const size_t tiles_n = N / Cfg::BN, tiles = tiles_n * div_ceil(M, Cfg::BM);  // < 2^31 / (BM * BN)
     const dim3 grid((unsigned)tiles, (unsigned)splits);
     HGEMM_CHECK(splits <= 65535);
@@ -144,7 +145,7 @@ void launch_splitk(const void *A, const void *B, void *C, size_t M, size_t N, si
     auto kernel = stream_b ? &hgemm_skinny_kernel<Cfg, true> : &hgemm_skinny_kernel<Cfg, false>;
     kernel<<<grid, dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
-        partial, (int)M, (int)N, (int)K, (int)(K / splits), (int)tiles_n);
+        partial, (int)M, (int)N, (int)K, splits, (int)tiles_n);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
     if (splits > 1) launch_splitk_reduce(partial, reinterpret_cast<half_t *>(C), M * N, splits);
 }
@@ -268,7 +269,7 @@ size_t padded_bytes(size_t M, size_t N, size_t K) {
 double predict_us(const Candidate &c, size_t M, size_t N, size_t K, int splits, size_t cus) {
     const size_t wgs = div_ceil(M, (size_t)c.bm) * div_ceil(N, (size_t)c.bn) * (size_t)splits;
     const size_t slots = cus * (size_t)c.per_cu;
-    const double chunks = (double)(K / (size_t)splits / 64);
+    const double chunks = (double)div_ceil(K / 64, (size_t)splits);  // the longest slice
     const size_t full = wgs / slots, rem = wgs % slots;
     double t = LAUNCH_US + (double)full * (c.fix + chunks * c.hi);
     if (rem) t += c.fix + chunks * (c.lo + (c.hi - c.lo) * (double)rem / (double)slots);
@@ -284,7 +285,7 @@ double predict_tail_us(const Candidate &c, size_t M, size_t N, size_t K, int ts,
     const size_t full = wgs / slots, rem = wgs % slots;
     const double chunks = (double)(K / 64);
     double t = LAUNCH_US + (double)full * (c.fix + chunks * c.hi);
-    t += LAUNCH_US + c.fix + chunks / ts * (c.lo + (c.hi - c.lo) * (double)(rem * ts) / (double)slots);
+    t += LAUNCH_US + c.fix + (double)div_ceil(K / 64, (size_t)ts) * (c.lo + (c.hi - c.lo) * (double)(rem * ts) / (double)slots);
     t += reduce_us(ts, (double)rem * c.bm * c.bn) + TAIL_US;
     return t;
 }
@@ -305,17 +306,35 @@ double predict_subtile_us(const Candidate &big, const Candidate &small, size_t M
     return t + TAIL_SUB_US;
 }
 
-// Number of K slices for `tiles` output tiles: the smallest power of two (<= 16) that
-// gives at least three quarters of the CUs a workgroup.  Each slice is a whole number of 64-wide chunks, at least
-// two of them.  (Measured on the decode shapes: more slices than that only add partial-sum
-// traffic, fewer leave CUs without a stream of B.)
+// Number of K slices (1 ... 16) for `tiles` output tiles of a split-K kernel, by a model of its time fitted to 91
+// shapes (M = 7 ... 128, N = 1408 ... 65536, K = 384 ... 15104, all five tiles) timed at every slice count on an MI355X,
+// operands rotated so that B streams from HBM:
+//     t(s) = t_B (1 + [s > 1] 8 s M / K) / balance(s) + [s > 1] 1 us,    t_B = 2 N K bytes at 5 TB/s,
+// balance(s) = w / (ceil(w / CUs) CUs) for w = tiles x s workgroups: the busiest CU runs ceil(w / CUs) of them, whether
+// side by side or one after the other, so 144 tiles run better in three slices (432 workgroups, two on most CUs) than
+// in two (288: two on a few CUs, one on the rest) -- M = 48, N = 9216, K = 8192: 43.8 / 45.0 / 35.8 / 41.9 us in 1 ... 4
+// slices.  The middle factor is the traffic of the fp32 partial sums (8 M bytes per slice and column of C, out and
+// back) against B's (2 K bytes per column), counted twice.  The model's choice is 1.2 % behind the best count on
+// average (16 % at worst); the rule it replaces (the smallest power of two that divides K's chunks and gives three
+// quarters of the CUs a workgroup) was 22 % behind on average.  A slice is a whole number of 64-wide chunks, at least
+// two; slices differ by at most one chunk.
 // `slice_bytes`: fp32 partial sums of one slice; the slices together stay within `limit`.
-int choose_splits(size_t tiles, size_t cus, size_t K, size_t slice_bytes, size_t limit) {
-    int s = 1;
-    while (s < 16 && tiles * s < cus * 3 / 4 && K % ((size_t)s * 2 * 64) == 0 && K / (s * 2) >= 128 &&
-           (size_t)(s * 2) * slice_bytes <= limit)
-        s *= 2;
-    return s;
+int choose_splits(size_t tiles, size_t M, size_t N, size_t cus, size_t K, size_t slice_bytes, size_t limit) {
+    int best = 1;
+    double best_us = 0.0;
+    const double stream_us = 2.0 * (double)N * (double)K / 5e6;
+    for (int s = 1; s <= 16; ++s) {
+        if (s > 1 && (K % 64 != 0 || K / 64 / (size_t)s < 2 || (size_t)s * slice_bytes > limit)) break;
+        const size_t wgs = tiles * (size_t)s;
+        const double balance = (double)wgs / (double)(div_ceil(wgs, cus) * cus);
+        const double partials = s > 1 ? 8.0 * s * (double)M / (double)K : 0.0;
+        const double us = stream_us * (1.0 + partials) / balance + (s > 1 ? 1.0 : 0.0);
+        if (s == 1 || us < best_us - 1e-9) {
+            best_us = us;
+            best = s;
+        }
+    }
+    return best;
 }
 
 
@@ -356,6 +375,20 @@ constexpr SmallMRule SMALL_M_RULES[] = {
     // kernel); below M = 6 and for smaller B the streaming kernel stays ahead.
     {6, 8, 1, ANY, 1, ANY, LARGE_B, ANY, 0, KERNEL_SPLIT_32x64},
     {1, 8, 1, ANY, 1, ANY, 0, ANY, 0, KERNEL_DECODE_BN16},
+    // --- M = 9 ... 24 against N >= 14336: the persistent kernel that keeps A in registers, where every wave can hold
+    // its slice of A (K = 512 ... 1536 per wave, eight waves; four waves of 1280 at K = 5120).  Against what ran these
+    // shapes before, over N = 14336 ... 57344: K = 6144 (split-K before) 1.06 ... 1.30x, K = 10240 and 12288 1.08 ... 1.40x,
+    // K = 5120 1.07 ... 1.31x from N = 18432 (0.96 ... 1.08x at 14336), K = 8192 (ring kernel) 1.03 ... 1.14x, K = 4096
+    // 1.04 ... 1.06x at M = 16 from N = 18432 (N = 28672: 40.1 -> 37.8 us) and level at M = 9, so from M = 13; M = 17 ... 24
+    // (two row tiles, 64x128 pipelined tile before) 1.09 ... 1.13x at N = 18432 and 57344 and 0.93 ... 1.09x at N = 28672
+    // depending on the box; M = 32 and K <= 3072 mixed (0.68 ... 1.2x), so not taken.
+    {9, 16, 18432, ANY, 5120, 5120, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
+    {9, 16, 14336, ANY, 10240, 10240, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
+    {9, 16, 14336, ANY, 12288, 12288, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
+    {9, 16, 14336, ANY, 6144, 6144, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
+    {9, 16, 14336, ANY, 8192, 8192, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
+    {13, 16, 18432, ANY, 4096, 4096, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
+    {17, 24, 18432, ANY, 4096, 4096, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
     // --- M = 9 ... 16: the ring kernel up to N = 8192 while K <= 4096 (K <= 8192 up to N = 4096); beyond, K slices
     // across workgroups are up to 29 % ahead -- except, with the non-temporal copies, against a B of 48 MB or more at
     // K = 2048, 4096 and 8192, where every wave walks 1024 of K (M = 12: 1.05 ... 1.29x, M = 16: 0.97 ... 1.23x over
@@ -414,6 +447,7 @@ bool small_m_rule_covers(const SmallMRule &r, size_t M, size_t N, size_t K) {
 bool small_m_kernel_supports(int kernel, size_t M, size_t N, size_t K) {
     switch (kernel) {
         case KERNEL_DECODE_RING: return decode_ring_supports(M, N, K);
+        case KERNEL_DECODE_RESIDENT: return decode_resident_supports(M, N, K);
         case KERNEL_DECODE_BN16: return decode_supports(M, N, K);
         case KERNEL_MID128:
         case KERNEL_ROW64x128: return N % 8 == 0 && K % 64 == 0 && K >= 64 * 5;
@@ -443,6 +477,11 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
         p.kernel = r.kernel;
         switch (r.kernel) {
             case KERNEL_DECODE_RING: p.splits = decode_ring_waves(M, N, K, cus); break;
+            case KERNEL_DECODE_RESIDENT: {
+                int chunks = 0;
+                p.splits = decode_resident_waves(M, K, &chunks);
+                break;
+            }
             case KERNEL_DECODE_BN16: {  // the streaming kernel: 16 or 32 columns per workgroup
                 int bn = 16, waves = 1;
                 decode_plan(M, N, K, cus, &bn, &waves);
@@ -451,10 +490,30 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
                 break;
             }
             case KERNEL_MID128:
-            case KERNEL_ROW64x128: p.splits = 1; break;
+            case KERNEL_ROW64x128: {
+                // One workgroup per CU.  More column tiles than CUs: the tiles beyond the whole rounds would run as a
+                // round of their own on a few CUs, so they are cut into K slices that fill the chip (M = 103,
+                // N = 34304, K = 6656: 268 tiles, 133 us as two rounds against 89 us for hipBLASLt).
+                p.splits = 1;
+                const size_t tiles = div_ceil(N, (size_t)128), rem = tiles % cus;
+                const size_t tile_bytes = (size_t)(r.kernel == KERNEL_MID128 ? 128 : 64) * 128 * sizeof(float);
+                if (tiles > cus && rem > 0) {
+                    size_t ts = cus / rem < 16 ? cus / rem : 16;
+                    while (ts >= 2 && (shortest_slice(K, 64, (int)ts) < 64 * 5 || ts * rem * tile_bytes > limits.partial_bytes)) --ts;
+                    // worth its extra launch and reduction (about 6 us) when the round it shortens is long: a round
+                    // takes about half a microsecond per chunk (M = 76, N = 39552, K = 640: 19.8 us as two rounds, 23.7
+                    // with the 53 tiles of the second in two slices)
+                    if (ts >= 2 && (double)(K / 64) * (1.0 - 1.0 / (double)ts) > 12.0) {
+                        p.tail_tiles = (int)rem;
+                        p.tail_splits = (int)ts;
+                        p.partial_bytes = ts * rem * tile_bytes;
+                    }
+                }
+                break;
+            }
             default: {  // the split-K family: K slices across workgroups, then the ordered reduction
                 const size_t bn = (r.kernel == KERNEL_SPLIT_64x128 || r.kernel == KERNEL_SPLIT_128x128) ? 128 : 64;
-                p.splits = choose_splits(N / bn, cus, K, slice_bytes, limits.partial_bytes);
+                p.splits = choose_splits(N / bn, M, N, cus, K, slice_bytes, limits.partial_bytes);
                 if (p.splits > 1) p.partial_bytes = (size_t)p.splits * slice_bytes;
             }
         }
@@ -467,7 +526,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
         if (N % 8) break;
         const bool whole_tiles_only = c.kernel == KERNEL_SMALL64_W4;
         if (whole_tiles_only && (M % c.bm || N % c.bn)) continue;
-        for (int s = 1; s <= 32; s *= 2) {
+        for (int s = 1; s <= 32; ++s) {  // K slices: whole chunks, as even as that allows
             if (whole_tiles_only) {
                 const size_t wgs = (M / c.bm) * (N / c.bn) * (size_t)s;
                 if (wgs > cus * (size_t)c.per_cu) break;
@@ -477,7 +536,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
             // whole 64x64 tiles, at most one workgroup per CU: the four-wave tile is ahead of the one-wave tile on
             // every such grid that was measured (the model, fitted on larger grids, flatters the one-wave tile there)
             if (c.kernel == KERNEL_SMALL64 && M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) * (size_t)s <= cus) continue;
-            if (K % ((size_t)s * 64) || K / s < (size_t)64 * c.stages) break;
+            if (K % 64 || shortest_slice(K, 64, s) < (size_t)64 * c.stages) break;
             if (s > 1 && (size_t)s * slice_bytes > limits.partial_bytes) break;
             const double t = predict_us(c, M, N, K, s, cus);
             if (p.kernel == KERNEL_NONE || t < best) {
@@ -495,8 +554,8 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
         const size_t wgs = div_ceil(M, (size_t)c.bm) * div_ceil(N, (size_t)c.bn), slots = cus * (size_t)c.per_cu;
         const size_t rem = wgs % slots;
         if (wgs > slots && rem > 0 && !whole_tiles_only && c.kernel != KERNEL_MID128_S2) {
-            for (int ts = 2; ts <= 16; ts *= 2) {
-                if (K % ((size_t)ts * 64) || K / ts < (size_t)64 * c.stages || rem * ts > slots) break;
+            for (int ts = 2; ts <= 16; ++ts) {
+                if (K % 64 || shortest_slice(K, 64, ts) < (size_t)64 * c.stages || rem * ts > slots) break;
                 if ((size_t)ts * rem * c.bm * c.bn * sizeof(float) > limits.partial_bytes) break;
                 const double t = predict_tail_us(c, M, N, K, ts, cus);
                 if (p.kernel != KERNEL_NONE && t < best) {
@@ -534,7 +593,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     if (p.kernel != KERNEL_NONE) return p;
     if (N % 64 == 0 && K % 64 == 0) {  // any M: rows beyond M are guarded
         p.kernel = KERNEL_SPLIT_64x64;
-        p.splits = choose_splits(div_ceil(M, 64) * (N / 64), cus, K, slice_bytes, limits.partial_bytes);
+        p.splits = choose_splits(div_ceil(M, 64) * (N / 64), M, N, cus, K, slice_bytes, limits.partial_bytes);
         if (p.splits > 1) p.partial_bytes = (size_t)p.splits * slice_bytes;
         return p;
     }
@@ -629,7 +688,7 @@ void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, 
         case KERNEL_R256x128: launch_pipelined_plan<Rect256x128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128_S2: launch_pipelined<Mid128S2>(A, B, C, M, N, K, "hgemm_auto"); break;
-        case KERNEL_ROW64x128: launch_pipelined<Row64x128>(A, B, C, M, N, K, "hgemm_auto"); break;
+        case KERNEL_ROW64x128: launch_pipelined_plan<Row64x128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_SMALL64_W4: {
             const size_t chunks = K / 64 / (size_t)(p.splits > 1 ? p.splits : 1);
@@ -663,6 +722,7 @@ void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, 
         case KERNEL_DECODE_BN16: launch_decode(A, B, C, M, N, K, 16, p.splits); break;
         case KERNEL_DECODE_BN32: launch_decode(A, B, C, M, N, K, 32, p.splits); break;
         case KERNEL_DECODE_RING: launch_decode_ring(A, B, C, M, N, K, p.splits); break;
+        case KERNEL_DECODE_RESIDENT: launch_decode_resident(A, B, C, M, N, K, compute_units()); break;
         case KERNEL_RAGGED: launch_ragged(A, B, C, M, N, K); break;
         case KERNEL_PADDED: run_padded(p, ws, A, B, C, M, N, K); break;
         case KERNEL_SIMT:
@@ -843,7 +903,7 @@ extern "C" int hgemm_auto_plan_tail_kernel(size_t M, size_t N, size_t K) { retur
 extern "C" int hgemm_auto_plan_chained(size_t M, size_t N, size_t K) {
     const Plan p = plan_for(M, N, K);
     if (p.splits < 1) return 0;
-    const size_t k_len = K / (size_t)p.splits;
+    const size_t k_len = shortest_slice(K, 64, p.splits);
     auto workgroups = [&](size_t bm, size_t bn) {  // of the main launch
         return (div_ceil(M, bm) * div_ceil(N, bn) - (size_t)p.tail_tiles) * (size_t)p.splits;
     };
@@ -872,6 +932,7 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
         case KERNEL_DECODE_BN16: return "streaming decode, 16 columns per workgroup, one wave per K slice";
         case KERNEL_DECODE_BN32: return "streaming decode, 32 columns per workgroup, one wave per K slice";
         case KERNEL_DECODE_RING: return "streaming decode, 16 columns per workgroup, one wave and one LDS ring per K slice";
+        case KERNEL_DECODE_RESIDENT: return "decode with A in registers, persistent workgroups over 16-column tiles, one wave per K slice";
         case KERNEL_RAGGED: return "guarded 128x128x32, 4 waves, any shape";
         case KERNEL_PADDED: return "zero-padded operand copies + pipelined kernel of the padded shape";
         case KERNEL_SIMT: return "scalar fallback";

@@ -119,7 +119,7 @@ __device__ __forceinline__ void store_chained_tile(unsigned char *lds, half_t *_
 template <class Cfg, bool SPLIT = false, bool EDGE = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_chained_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
-                           float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n,
+                           float *__restrict__ partial, int M, int N, int K, int slices, int tiles_m, int tiles_n,
                            int first_block, int tail_tiles, int subdiv) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
     constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS;
@@ -133,7 +133,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
     PipeFrame<Cfg, SPLIT, EDGE> frame;
-    if (!frame.init(A, B, M, N, K, k_len, tiles_m, tiles_n, first_block, subdiv, lds_base)) return;
+    if (!frame.init(A, B, M, N, K, slices, tiles_m, tiles_n, first_block, subdiv, lds_base)) return;
     const int lane = frame.lane, wave = frame.wave, wm = frame.wm, wn = frame.wn;
     int tile_m = frame.tile_m, tile_n = frame.tile_n;
     const int slot = frame.slot, slice = frame.slice, num_k = frame.num_k;

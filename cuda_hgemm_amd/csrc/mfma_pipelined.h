@@ -313,7 +313,7 @@ struct PipeFrame {
     uint32_t a_addr[KSTEPS][NF], b_addr[KSTEPS][NF];
 
     // false: this workgroup has no tile (a part of a subdivided tile that lies wholly outside the matrix)
-    __device__ __forceinline__ bool init(const half_t *A, const half_t *B, int M, int N, int K, int k_len, int tiles_m,
+    __device__ __forceinline__ bool init(const half_t *A, const half_t *B, int M, int N, int K, int slices, int tiles_m,
                                          int tiles_n, int first_block, int subdiv, uint32_t lds_base) {
         const int tid = threadIdx.x;
         lane = tid & 63;
@@ -325,7 +325,6 @@ struct PipeFrame {
         // that those neighbours also work on the same slice of K.
         slice = 0;
         if constexpr (SPLIT) {
-            const int slices = K / k_len;
             slice_and_slot_of_workgroup((int)blockIdx.x, (int)gridDim.x / slices, slices, slice, slot);
             slice = __builtin_amdgcn_readfirstlane(slice);
         } else {
@@ -347,8 +346,9 @@ struct PipeFrame {
         }
         tile_m = __builtin_amdgcn_readfirstlane(tile_m);  // wave-uniform by construction: keep them in SGPRs
         tile_n = __builtin_amdgcn_readfirstlane(tile_n);
-        num_k = k_len / BK;
-        const int k_begin = slice * k_len;
+        int first_chunk;
+        slice_of_k(K / BK, slices, slice, first_chunk, num_k);
+        const int k_begin = first_chunk * BK;
 
         // ---- copies: wave w, instruction i fills LDS rows [(i*WAVES + w)*ROWS_PER_DMA, +ROWS_PER_DMA)
         a_base = reinterpret_cast<const unsigned char *>(A + (size_t)tile_m * BM * K + k_begin);
@@ -412,7 +412,7 @@ struct PipeFrame {
 template <class Cfg, bool SPLIT = false, bool EDGE = false, bool STREAM_B = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_pipelined_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
-                           float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n,
+                           float *__restrict__ partial, int M, int N, int K, int slices, int tiles_m, int tiles_n,
                            int first_block, int tail_tiles, int subdiv) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, MI = Cfg::MI;
     constexpr int TM = Cfg::PTM, TN = Cfg::PTN, KSTEPS = Cfg::PKSTEPS;
@@ -427,7 +427,7 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
     PipeFrame<Cfg, SPLIT, EDGE> frame;
-    if (!frame.init(A, B, M, N, K, k_len, tiles_m, tiles_n, first_block, subdiv, lds_base)) return;
+    if (!frame.init(A, B, M, N, K, slices, tiles_m, tiles_n, first_block, subdiv, lds_base)) return;
     const int lane = frame.lane, wave = frame.wave, wm = frame.wm, wn = frame.wn;
     const int tile_m = frame.tile_m, tile_n = frame.tile_n, slot = frame.slot, slice = frame.slice;
     const int num_k = frame.num_k;
@@ -786,17 +786,16 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
         if (which != PipeKernel::Chained && stream_b_pays(tiles_m, N, K)) {
             hgemm_pipelined_kernel<Cfg, SPLIT, EDGE, true><<<dim3(blocks), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
                 reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
-                partial, (int)M, (int)N, (int)K, (int)K, tiles_m, tiles_n, first_block, tail_tiles, subdiv);
+                partial, (int)M, (int)N, (int)K, 1, tiles_m, tiles_n, first_block, tail_tiles, subdiv);
             HGEMM_CHECK_HIP_ERROR(hipGetLastError());
             return;
         }
     }
     if constexpr (chained_available<Cfg>()) {
-        if (use_chained<Cfg>(which, (size_t)blocks * (size_t)splits, K / (size_t)splits)) {
+        if (use_chained<Cfg>(which, (size_t)blocks * (size_t)splits, shortest_slice(K, Cfg::BK, splits))) {
             hgemm_chained_kernel<Cfg, SPLIT, EDGE><<<dim3(blocks * splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
                 reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
-                partial, (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, first_block, tail_tiles,
-                subdiv);
+                partial, (int)M, (int)N, (int)K, splits, tiles_m, tiles_n, first_block, tail_tiles, subdiv);
             HGEMM_CHECK_HIP_ERROR(hipGetLastError());
             return;
         }
@@ -804,7 +803,7 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
     HGEMM_CHECK_MSG(which != PipeKernel::Chained, "this tile has no chained kernel");
     hgemm_pipelined_kernel<Cfg, SPLIT, EDGE><<<dim3(blocks * splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), partial,
-        (int)M, (int)N, (int)K, (int)(K / (size_t)splits), tiles_m, tiles_n, first_block, tail_tiles, subdiv);
+        (int)M, (int)N, (int)K, splits, tiles_m, tiles_n, first_block, tail_tiles, subdiv);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 
@@ -818,9 +817,9 @@ void launch_pipelined_with_tail(const void *A, const void *B, void *C, float *pa
     check_operands(A, B, C, M, N, K);
     const int tiles_m = (int)div_ceil(M, (size_t)Cfg::BM), tiles_n = (int)div_ceil(N, (size_t)Cfg::BN);
     const int total = tiles_m * tiles_n, head = total - tail_tiles;
-    HGEMM_CHECK(partial != nullptr && tail_tiles >= 1 && head >= 1 && tail_splits >= 2 && K % (size_t)tail_splits == 0);
-    HGEMM_CHECK_MSG(pipelined_supports_edges<Cfg>(M, N, K / (size_t)tail_splits),
-                    "%s (tail in %d K slices) needs N %% 8 == 0, slice %% %d == 0, slice >= %d (got M=%zu N=%zu K=%zu)",
+    HGEMM_CHECK(partial != nullptr && tail_tiles >= 1 && head >= 1 && tail_splits >= 2 && K % (size_t)Cfg::BK == 0);
+    HGEMM_CHECK_MSG(pipelined_supports_edges<Cfg>(M, N, shortest_slice(K, Cfg::BK, tail_splits)),
+                    "%s (tail in %d K slices) needs N %% 8 == 0, K %% %d == 0, shortest slice >= %d (got M=%zu N=%zu K=%zu)",
                     name, tail_splits, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
     if (Cfg::supports(M, N, K)) {
         launch_pipelined_impl<Cfg, false, false>(A, B, C, nullptr, M, N, K, 1, 0, head);
@@ -856,14 +855,14 @@ void launch_pipelined(const void *A, const void *B, void *C, size_t M, size_t N,
 template <class Cfg>
 void launch_pipelined_split(const void *A, const void *B, float *partial, size_t M, size_t N, size_t K, int splits,
                             const char *name) {
-    HGEMM_CHECK(splits >= 1 && K % (size_t)splits == 0 && partial != nullptr);
-    const size_t k_len = K / (size_t)splits;
-    if (Cfg::supports(M, N, k_len)) {
+    HGEMM_CHECK(splits >= 1 && K % (size_t)Cfg::BK == 0 && partial != nullptr);
+    const size_t k_len = shortest_slice(K, Cfg::BK, splits);
+    if (k_len > 0 && Cfg::supports(M, N, k_len)) {
         launch_pipelined_impl<Cfg, true, false>(A, B, nullptr, partial, M, N, K, splits);
         return;
     }
-    HGEMM_CHECK_MSG(pipelined_supports_edges<Cfg>(M, N, k_len),
-                    "%s (K in %d slices) needs N %% 8 == 0, slice %% %d == 0, slice >= %d (got M=%zu N=%zu K=%zu)",
+    HGEMM_CHECK_MSG(k_len > 0 && pipelined_supports_edges<Cfg>(M, N, k_len),
+                    "%s (K in %d slices) needs N %% 8 == 0, K %% %d == 0, shortest slice >= %d (got M=%zu N=%zu K=%zu)",
                     name, splits, Cfg::BK, Cfg::BK * Cfg::STAGES, M, N, K);
     launch_pipelined_impl<Cfg, true, true>(A, B, nullptr, partial, M, N, K, splits);
 }
@@ -901,7 +900,7 @@ void launch_pipelined_with_subtiles(const void *A, const void *B, void *C, size_
     (void)configured;
     kernel<<<dim3(tail_tiles * sub_m * sub_n), dim3(Child::THREADS), Child::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), nullptr,
-        (int)M, (int)N, (int)K, (int)K, tiles_m, tiles_n, head, 0, (sub_m << 8) | sub_n);
+        (int)M, (int)N, (int)K, 1, tiles_m, tiles_n, head, 0, (sub_m << 8) | sub_n);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 

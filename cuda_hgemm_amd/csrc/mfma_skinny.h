@@ -28,7 +28,7 @@ struct SkinnyConfig : TileConfig<BM_, BN_, 64, WAVES_M_, WAVES_N_, STAGES_, LOAD
 template <class Cfg, bool STREAM_B = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_skinny_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
-                        float *__restrict__ partial, int M, int N, int K, int k_per_split, int tiles_n) {
+                        float *__restrict__ partial, int M, int N, int K, int splits, int tiles_n) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, KSTEPS = Cfg::KSTEPS, CPR = Cfg::CPR;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES;
@@ -44,8 +44,9 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     // grid: x = tiles of C, row-major (no 65535 limit on the number of row or column tiles), y = K slice
     const int tile_n = (int)blockIdx.x % tiles_n, tile_m = (int)blockIdx.x / tiles_n, split = blockIdx.y;
     const int m0 = tile_m * BM;
-    const int k_begin = split * k_per_split;
-    const int num_k = k_per_split / BK;
+    int first_chunk, num_k;  // K's chunks are dealt to the slices as evenly as whole chunks allow
+    slice_of_k(K / BK, splits, split, first_chunk, num_k);
+    const int k_begin = first_chunk * BK;
 
     // ---- copy set-up (rows of A clamped to the last valid row)
     constexpr int DMA_ROW_STEP = Cfg::WAVES * Cfg::ROWS_PER_DMA;

@@ -88,6 +88,16 @@ struct TileConfig {
     }
 };
 
+// K in slices of whole chunks, as even as that allows: the first `chunks % slices` slices walk one chunk more.
+// Slice `slice` starts at chunk `first` and walks `count`.
+__host__ __device__ __forceinline__ void slice_of_k(int chunks, int slices, int slice, int &first, int &count) {
+    const int base = chunks / slices, longer = chunks % slices;
+    first = slice * base + (slice < longer ? slice : longer);
+    count = base + (slice < longer ? 1 : 0);
+}
+// the length of the shortest of `splits` such slices of K (chunks of `bk`), which is what a kernel's minimum K applies to
+inline size_t shortest_slice(size_t K, int bk, int splits) { return K / (size_t)bk / (size_t)splits * (size_t)bk; }
+
 // s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left at "do not wait"); gfx9 encoding.
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -202,13 +212,13 @@ __device__ __forceinline__ void store_tile_via_lds(const floatx16 (&acc)[Cfg::TM
     }
 }
 
-// SPLIT: a one-dimensional launch of tiles x slices workgroups; each computes one K slice (k_len wide) of one tile
-// and leaves fp32 partial sums in partial[slice][M][N] for the ordered reduction; otherwise k_len == K and C is
-// written.
+// SPLIT: a one-dimensional launch of tiles x slices workgroups; each computes one K slice of one tile and leaves
+// fp32 partial sums in partial[slice][M][N] for the ordered reduction; otherwise slices == 1 and C is written.
+// The K / BK chunks are dealt to the slices as evenly as whole chunks allow (`slice_of_k`).
 template <class Cfg, bool SPLIT = false>
 __global__ void __launch_bounds__(Cfg::THREADS)
     hgemm_tiled_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, half_t *__restrict__ C,
-                       float *__restrict__ partial, int M, int N, int K, int k_len, int tiles_m, int tiles_n) {
+                       float *__restrict__ partial, int M, int N, int K, int slices, int tiles_m, int tiles_n) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, KSTEPS = Cfg::KSTEPS, CPR = Cfg::CPR;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, STAGES = Cfg::STAGES, THREADS = Cfg::THREADS;
@@ -224,17 +234,18 @@ __global__ void __launch_bounds__(Cfg::THREADS)
     int tile_m, tile_n, slice = 0;
     if constexpr (SPLIT) {
         int slot;
-        slice_and_slot_of_workgroup((int)blockIdx.x, tiles_m * tiles_n, K / k_len, slice, slot);
+        slice_and_slot_of_workgroup((int)blockIdx.x, tiles_m * tiles_n, slices, slice, slot);
         tile_of_position(blocked_order(N, K), slot, tiles_m, tiles_n, tile_m, tile_n);
         slice = __builtin_amdgcn_readfirstlane(slice);
     } else {
         tile_of_workgroup(blocked_order(N, K), 0, (int)blockIdx.x, (int)gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
     }
 
-    const int k_begin = slice * k_len;
+    int first_chunk, num_k;
+    slice_of_k(K / BK, slices, slice, first_chunk, num_k);
+    const int k_begin = first_chunk * BK;
     const half_t *Ag = A + (size_t)tile_m * BM * K + k_begin;
     const half_t *Bg = B + (size_t)tile_n * BN * K + k_begin;
-    const int num_k = k_len / BK;
 
     // ---------------- global -> LDS copy set-up ----------------
     // REG: thread t moves chunk (row = t / CPR + it * THREADS/CPR, ch = t % CPR).
@@ -501,7 +512,7 @@ void launch_tiled(const void *A, const void *B, void *C, size_t M, size_t N, siz
     const int tiles_m = (int)(M / Cfg::BM), tiles_n = (int)(N / Cfg::BN);
     hgemm_tiled_kernel<Cfg><<<dim3(tiles_m * tiles_n), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C), nullptr,
-        (int)M, (int)N, (int)K, (int)K, tiles_m, tiles_n);
+        (int)M, (int)N, (int)K, 1, tiles_m, tiles_n);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 
@@ -509,10 +520,10 @@ void launch_tiled(const void *A, const void *B, void *C, size_t M, size_t N, siz
 template <class Cfg>
 void launch_tiled_split(const void *A, const void *B, float *partial, size_t M, size_t N, size_t K, int splits,
                         const char *name) {
-    HGEMM_CHECK(splits >= 1 && K % (size_t)splits == 0 && partial != nullptr && splits <= 65535);
-    const size_t k_len = K / (size_t)splits;
-    HGEMM_CHECK_MSG(Cfg::supports(M, N, k_len),
-                    "%s (K in %d slices) needs M %% %d == 0, N %% %d == 0, slice %% %d == 0, slice >= %d (got M=%zu N=%zu K=%zu)",
+    HGEMM_CHECK(splits >= 1 && K % (size_t)Cfg::BK == 0 && partial != nullptr && splits <= 65535);
+    const size_t k_len = shortest_slice(K, Cfg::BK, splits);
+    HGEMM_CHECK_MSG(k_len > 0 && Cfg::supports(M, N, k_len),
+                    "%s (K in %d slices) needs M %% %d == 0, N %% %d == 0, K %% %d == 0, shortest slice >= %d (got M=%zu N=%zu K=%zu)",
                     name, splits, Cfg::BM, Cfg::BN, Cfg::BK, Cfg::BK * (Cfg::STAGES > 1 ? Cfg::STAGES - 1 : 1), M, N, K);
     static bool configured = [] {
         HGEMM_CHECK_HIP_ERROR(hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_tiled_kernel<Cfg, true>),
@@ -524,7 +535,7 @@ void launch_tiled_split(const void *A, const void *B, float *partial, size_t M, 
     HGEMM_CHECK((size_t)tiles_m * tiles_n * (size_t)splits < ((size_t)1 << 31));
     hgemm_tiled_kernel<Cfg, true><<<dim3(tiles_m * tiles_n * splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
         reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), nullptr, partial, (int)M, (int)N, (int)K,
-        (int)k_len, tiles_m, tiles_n);
+        splits, tiles_m, tiles_n);
     HGEMM_CHECK_HIP_ERROR(hipGetLastError());
 }
 

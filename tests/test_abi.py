@@ -107,7 +107,9 @@ def test_auto_plan_covers_every_benchmark_config(hgemm_lib):
     for m in (1, 8, 16, 64, 128):
         for n in (4096, 28672):
             p = plan(m, n, 4096)
-            if m <= 16:      # the decode kernel with per-wave LDS rings (B copied non-temporally at N = 28672)
+            if m == 16 and n == 28672:   # A in registers, persistent workgroups, eight K slices of 512 per workgroup
+                assert p["kernel"].startswith("decode with A in registers") and p["splits"] == 8, (m, n, p)
+            elif m <= 16:    # the decode kernel with per-wave LDS rings (B copied non-temporally at N = 28672)
                 assert "LDS ring per K slice" in p["kernel"] and p["splits"] == 4, (m, n, p)
             elif n == 28672:                                # one tile row against 224 column tiles: one launch
                 assert p["kernel"].startswith("pipelined %dx128x64" % m) and p["splits"] == 1, (m, n, p)
@@ -136,6 +138,9 @@ def test_small_m_rule_table(hgemm_lib):
         assert last["n_hi"] > 1 << 40 and last["k_hi"] > 1 << 40 and not last["k_below_4n"], (m, last)
 
     def can_run(kernel, M, N, K):
+        if kernel.startswith("decode with A in registers"):      # K = waves x chunks x 64, the chunks in registers
+            chunk_options = (8,) if M > 16 else (8, 12, 16, 20, 24)
+            return M <= 32 and N % 16 == 0 and K % 64 == 0 and any(K // 64 == w * c for w in (2, 4, 8) for c in chunk_options)
         if "LDS ring per K slice" in kernel:
             return N % 16 == 0 and K % 128 == 0
         if kernel.startswith("streaming decode"):
@@ -160,9 +165,9 @@ def test_small_m_rule_table(hgemm_lib):
 
     family = lambda name: name.split(",")[0].replace("32 columns", "16 columns")   # the streaming kernel's two widths
     checked = 0
-    for M in (1, 5, 6, 8, 9, 16, 17, 24, 25, 32, 33, 64, 65, 100, 128):    # both sides of every M class boundary
+    for M in (1, 5, 6, 8, 9, 12, 13, 16, 17, 24, 25, 32, 33, 64, 65, 100, 128):    # both sides of every M class boundary
         for N in (16, 48, 64, 272, 2048, 3072, 4096, 4112, 8192, 8208, 14336, 16384, 18432, 20488, 28672, 57344):
-            for K in (64, 256, 384, 512, 1024, 1152, 2048, 2304, 4096, 4160, 8192, 12288, 16384, 32768):
+            for K in (64, 256, 384, 512, 1024, 1152, 2048, 2304, 4096, 4160, 6144, 8192, 12288, 16384, 32768):
                 expect = lookup(M, N, K)
                 if expect is None:
                     continue
@@ -173,13 +178,15 @@ def test_small_m_rule_table(hgemm_lib):
     # the headline decode shapes, by row
     assert lookup(1, 4096, 4096).endswith("one LDS ring per K slice") and lookup(128, 4096, 4096).startswith("split-K 128x64")
     assert lookup(1, 28672, 4096).endswith("one LDS ring per K slice") and lookup(128, 28672, 4096).startswith("pipelined 128x128")
-    assert lookup(64, 28672, 4096).startswith("pipelined 64x128") and lookup(16, 28672, 4096).endswith("one LDS ring per K slice")
+    assert lookup(64, 28672, 4096).startswith("pipelined 64x128") and lookup(8, 28672, 4096).endswith("one LDS ring per K slice")
+    assert lookup(16, 28672, 4096).startswith("decode with A in registers") and lookup(12, 28672, 4096).endswith("one LDS ring per K slice")
     assert lookup(16, 28672, 3072).startswith("split-K 32x64") and lookup(2, 28672, 512).startswith("streaming decode, 16")
 
 
 def test_auto_plan_invariants_over_many_shapes(hgemm_lib):
     """What run_plan relies on, for every plan the model can come up with (no launch, no GPU): K slices are whole
-    numbers of 64-wide chunks and fit the workspace cap; the four-wave 64x64 tile only takes grids of whole tiles, at
+    numbers of 64-wide chunks (the slices of a launch differ by at most one chunk), each at least as long as the
+    shortest K its kernel takes, and fit the workspace cap; the four-wave 64x64 tile only takes grids of whole tiles, at
     most two per CU, and is unsliced and below 40 chunks when two share a CU; the 2-stage 128x128 tile only takes
     K <= 256, unsliced, without a tail."""
     import random
@@ -195,18 +202,28 @@ def test_auto_plan_invariants_over_many_shapes(hgemm_lib):
         s = p["splits"]
         assert s >= 1 and p["tail_splits"] >= 1, (m, n, k, p)
         if p["kernel"].startswith(("pipelined", "tiled", "split-K")):
-            assert k % (64 * s) == 0 and k % (64 * p["tail_splits"]) == 0, (m, n, k, p)
+            shortest = {"pipelined 256x256": 2, "pipelined 192x192": 3, "pipelined 256x128": 3, "pipelined 128x128": 5,
+                        "pipelined 64x128": 5, "pipelined 64x64": 3, "tiled 64x64x64": 3, "split-K": 1}
+            floor = [v for key, v in shortest.items() if p["kernel"].startswith(key)][0]
+            if "2-stage ring" in p["kernel"]:
+                floor = 2
+            assert k % 64 == 0 and k // 64 // s >= (floor if s > 1 or not p["kernel"].startswith("split-K") else 1), (m, n, k, p)
+            assert k // 64 // p["tail_splits"] >= (floor if p["tail_splits"] > 1 else 1), (m, n, k, p)
         need = hgemm_lib.auto_workspace_bytes(m, n, k)
         assert need["partial"] <= 512 << 20 and need["operands"] <= 1024 << 20, (m, n, k, need)
         if p["kernel"].startswith("tiled 64x64x64"):
             assert m % 64 == 0 and n % 64 == 0 and p["tail_tiles"] == 0, (m, n, k, p)
             tiles = (m // 64) * (n // 64)
-            assert tiles * s <= 2 * cus and k // s >= 192, (m, n, k, p)
+            assert tiles * s <= 2 * cus and k // 64 // s >= 3, (m, n, k, p)
             if tiles * s > cus:
                 assert s == 1 and k // 64 < 40, (m, n, k, p)
         if "2-stage ring" in p["kernel"]:
             assert k <= 256 and s == 1 and p["tail_tiles"] == 0, (m, n, k, p)
-        if "LDS ring per K slice" in p["kernel"]:
+        if p["kernel"].startswith("decode with A in registers"):
+            # eight (four, two) waves, each with 8 ... 24 chunks of A in registers; rings and partial sums fit a CU
+            assert m <= 32 and n % 16 == 0 and s in (2, 4, 8) and k % (64 * s) == 0 and k // (64 * s) in (8, 12, 16, 20, 24), (m, n, k, p)
+            assert need == {"partial": 0, "operands": 0} and s * 8192 + 2 * s * (2 if m > 16 else 1) * 1024 <= 160 << 10, (m, n, k, p)
+        elif "LDS ring per K slice" in p["kernel"]:
             # whole 64-wide chunks per wave; the waves' rings (16, 24, 30, 54 KB for 1, 2, 4, 8 row tiles of A) fit a CU
             assert m <= 128 and n % 16 == 0 and k % (64 * s) == 0 and need == {"partial": 0, "operands": 0}, (m, n, k, p)
             ring_kb = 16 if m <= 16 else 24 if m <= 32 else 30 if m <= 64 else 54

@@ -282,6 +282,42 @@ def test_auto_every_tile_with_and_without_k_slices(oracle, hgemm_lib, gpu, shape
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), ref)
 
 
+@pytest.mark.parametrize("shape,kernel,where", [
+    ((227, 128, 1216), "pipelined 64x64x64", "main"), ((2531, 256, 3392), "pipelined 128x128x64", "main"),
+    ((131, 4096, 9536), "pipelined 192x192x64", "main"), ((320, 6272, 12352), "pipelined 192x192x64", "main chained"),
+    ((2900, 264, 11072), "pipelined 256x128x64", "main"), ((2089, 1024, 12608), "pipelined 256x128x64", "main chained"),
+    ((1075, 4120, 5632), "pipelined 256x256x64", "main chained"), ((192, 128, 1408), "tiled 64x64x64", "main"),
+    ((256, 256, 16384), "tiled 64x64x64", "main"), ((512, 8280, 4864), "pipelined 128x128x64", "tail"),
+    ((1024, 8240, 3264), "pipelined 256x128x64", "tail"), ((1024, 8840, 4288), "pipelined 256x128x64", "tail chained"),
+    ((640, 28672, 8192), "pipelined 256x256x64", "tail chained"),
+    ((1, 192, 1344), "split-K 32x64x64", "main"), ((63, 64, 1216), "split-K 64x64x64", "main"),
+    ((37, 17152, 2176), "split-K 64x128x64", "main"), ((80, 64, 1088), "split-K 128x64x64", "main"),
+    ((102, 16384, 1856), "split-K 128x128x64", "main"), ((110, 3072, 10112), "split-K 128x64x64", "main")])
+def test_k_slices_that_differ_by_a_chunk(oracle, hgemm_lib, gpu, shape, kernel, where):
+    """K is cut into slices of whole 64-wide chunks, as even as that allows: where the slice count does not divide the
+    chunk count the first slices walk one chunk more.  Every kernel that takes K slices (each pipelined tile,
+    interleaved and chained, the four-wave 64x64 tile, the last round of a large grid, the five split-K tiles), on a
+    shape whose plan has such slices."""
+    M, N, K = shape
+    plan = hgemm_lib.auto_plan(M, N, K)
+    slices = plan["tail_splits"] if where.startswith("tail") else plan["splits"]
+    assert plan["kernel"].startswith(kernel) and slices > 1 and (K // 64) % slices != 0, plan
+    assert bool(plan["chained"]) == where.endswith("chained"), plan
+    assert (plan["tail_tiles"] > 0) == where.startswith("tail"), plan
+    A, B = oracle.fill((M, K), 81, 1), oracle.fill((N, K), 81, 2)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    assert np.array_equal(first, second)
+    At, Bt = oracle.fill((M, K), 82, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 82, 2, oracle.TERNARY, 0, 1)
+    exact = _run(hgemm_lib, "hgemm_auto", At, Bt, gpu)
+    if M * N * K <= 3e10:
+        _assert_close(oracle, first, oracle.hgemm(A, B), K)
+        assert np.array_equal(exact, oracle.hgemm(At, Bt))
+    else:                                      # complete rows from every row of tiles
+        _sampled_check(oracle, first, A, B, K, rows_per_slab=16, slabs=6, seed=5)
+        for m0 in list(range(0, M - 16, 131)) + [M - 8]:
+            assert np.array_equal(exact[m0:m0 + 8], oracle.hgemm_rows(At, Bt, m0, 8)), m0
+
+
 @pytest.mark.parametrize("t", [768, 1280, 1536, 1792, 2048, 2304])
 @pytest.mark.parametrize("K", [7168, 10240, 13312, 16384])
 def test_auto_deep_k_plans(oracle, hgemm_lib, gpu, t, K):
@@ -378,7 +414,7 @@ def test_streaming_decode_kernel(oracle, hgemm_lib, gpu, shape):
                                    (16, 4096, 256), (64, 8192, 896), (33, 272, 384), (9, 1040, 640),
                                    (65, 4096, 1024), (128, 8192, 512), (100, 272, 384), (128, 4096, 256), (24, 4096, 4096), (5, 1040, 384), (8, 4096, 640),
                                    # B of 48 MB or more: the copies of B carry the non-temporal hint
-                                   (1, 28672, 4096), (8, 28672, 4096), (16, 28672, 4096), (5, 14336, 4096), (12, 16384, 8192),
+                                   (1, 28672, 4096), (8, 28672, 4096), (12, 28672, 4096), (5, 14336, 4096), (12, 12288, 8192),
                                    (3, 57344, 1024), (7, 28672, 2048), (8, 20480, 2816), (6, 14336, 4096), (16, 8192, 4096)])
 def test_decode_kernel_with_lds_rings(oracle, hgemm_lib, gpu, shape):
     """M <= 128 through per-wave LDS rings (one, two, four or eight 16-row tiles of A per wave): one, two, four and eight K slices per workgroup, slices of one chunk and of
@@ -393,6 +429,25 @@ def test_decode_kernel_with_lds_rings(oracle, hgemm_lib, gpu, shape):
     _assert_close(oracle, first, oracle.hgemm(A, B), K)
     assert np.array_equal(first, second)
     At, Bt = oracle.fill((M, K), 36, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 36, 2, oracle.TERNARY, 0, 1)
+    assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
+
+
+@pytest.mark.parametrize("shape", [(16, 28672, 4096), (13, 18448, 4096), (9, 14336, 6144), (16, 14336, 8192), (11, 14352, 8192),
+                                   (17, 18432, 4096), (24, 20496, 4096), (20, 57344, 4096), (14, 16384, 6144)])
+def test_decode_kernel_with_a_in_registers(oracle, hgemm_lib, gpu, shape):
+    """M = 9 ... 24 against N >= 14336: persistent workgroups that load their waves' K slices of A into registers once
+    and walk over 16-column tiles of C.  8, 12 and 16 chunks of K per wave, one and two row tiles of A, one and two
+    workgroups per CU, tile counts that do and do not divide among the workgroups (some get one tile more; with 897
+    tiles and 512 workgroups some get a single tile), rows of A beyond M."""
+    M, N, K = shape
+    plan = hgemm_lib.auto_plan(M, N, K)
+    assert plan["kernel"].startswith("decode with A in registers") and plan["splits"] == 8, plan
+    A = oracle.fill((M, K), 37, 1, oracle.NORMAL, 0.0, 1.0)
+    B = oracle.fill((N, K), 37, 2, oracle.NORMAL, 0.0, 0.02)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    _assert_close(oracle, first, oracle.hgemm(A, B), K)
+    assert np.array_equal(first, second)
+    At, Bt = oracle.fill((M, K), 38, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 38, 2, oracle.TERNARY, 0, 1)
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
@@ -414,14 +469,14 @@ def test_small_m_against_a_large_b(oracle, hgemm_lib, gpu, shape):
 @pytest.mark.parametrize("shape", [(128, 28672, 4096), (100, 18440, 1024), (65, 20480, 2048), (128, 18432, 1088),
                                    (97, 24584, 1024), (128, 28672, 320 + 704),
                                    (64, 28672, 4096), (33, 18440, 1024), (50, 20480, 2048), (64, 24584, 1088), (64, 28672, 320),
-                                   (128, 28672, 384), (17, 28672, 4096), (32, 18432, 8192)])
+                                   (128, 28672, 384), (25, 28672, 4096), (32, 18432, 8192)])
 def test_one_tile_row_against_many_column_tiles(oracle, hgemm_lib, gpu, shape):
     """M = 33 ... 128 against N >= 18432: one launch of the pipelined kernel on a 128x128 tile (a 64x128 tile up to
     M = 64) whose copies of B carry the non-temporal hint (from 48 MB of B on; the smaller cases run the same rule
     without the hint), rows of the tile beyond M and a last column tile that ends inside the tile included."""
     M, N, K = shape
     plan = hgemm_lib.auto_plan(M, N, K)
-    tile = "128x128x64" if M > 64 else "64x128x64"      # M = 17 ... 32 join the 64x128 tile from K = 4096
+    tile = "128x128x64" if M > 64 else "64x128x64"      # M = 25 ... 32 (at K = 8192: 17 ... 32) join the 64x128 tile from K = 4096
     assert plan["kernel"].startswith(f"pipelined {tile}, 4 waves, 5-stage") and plan["splits"] == 1, plan
     A = oracle.fill((M, K), 41, 1, oracle.NORMAL, 0.0, 1.0)
     B = oracle.fill((N, K), 41, 2, oracle.NORMAL, 0.0, 0.02)
@@ -429,6 +484,26 @@ def test_one_tile_row_against_many_column_tiles(oracle, hgemm_lib, gpu, shape):
     _assert_close(oracle, first, oracle.hgemm(A, B), K)
     assert np.array_equal(first, second)
     At, Bt = oracle.fill((M, K), 42, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 42, 2, oracle.TERNARY, 0, 1)
+    assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
+
+
+@pytest.mark.parametrize("shape,tail", [((103, 34304, 6656), (12, 16)), ((117, 39936, 1600), (56, 4)), ((50, 33024, 2048), (2, 6)),
+                                        ((128, 65792, 2112), (2, 6)), ((64, 32776, 4096), (1, 12)), ((76, 39552, 640), (0, 1))])
+def test_one_tile_row_with_more_tiles_than_cus(oracle, hgemm_lib, gpu, shape, tail):
+    """One row of 128x128 or 64x128 tiles against more column tiles than the chip has CUs: whole rounds in one launch
+    (B copied non-temporally), the tiles beyond them in K slices that fill the chip, slices that differ by a chunk
+    and a last tile that ends inside N included; with a short K the tiles beyond the whole rounds stay a round of
+    their own."""
+    M, N, K = shape
+    plan = hgemm_lib.auto_plan(M, N, K)
+    assert plan["kernel"].startswith("pipelined %s" % ("128x128x64" if M > 64 else "64x128x64")) and plan["splits"] == 1, plan
+    assert (plan["tail_tiles"], plan["tail_splits"]) == tail and plan["tail_kernel"] == "none", plan
+    A = oracle.fill((M, K), 43, 1, oracle.NORMAL, 0.0, 1.0)
+    B = oracle.fill((N, K), 43, 2, oracle.NORMAL, 0.0, 0.02)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    _assert_close(oracle, first, oracle.hgemm(A, B), K)
+    assert np.array_equal(first, second)
+    At, Bt = oracle.fill((M, K), 44, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 44, 2, oracle.TERNARY, 0, 1)
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
