@@ -166,6 +166,8 @@ using Mid128S2 = PipeConfig<128, 128, 64, 2, 2, 2, 16>;
 using Small64 = PipeConfig<64, 64, 64, 1, 1, 3, 16>;
 // one row of tiles for M <= 64: four waves side by side, 64x32 each
 using Row64x128 = PipeConfig<64, 128, 64, 1, 4, 5, 16>;
+// one row of tiles for M = 129 ... 192: four stages of 24 + 16 KB are the whole LDS
+using Row192x128 = PipeConfig<192, 128, 64, 2, 2, 4, 16>;
 using Tile192 = PipeConfig<192, 192, 64, 2, 2, 3, 16>;
 using Rect256x128 = PipeConfig<256, 128, 64, 2, 2, 3, 16>;
 // 64x64x64 on four waves (one 32x32 MFMA tile each) with the ladder's kernel: a small tile whose chunk takes a quarter
@@ -457,6 +459,24 @@ bool small_m_kernel_supports(int kernel, size_t M, size_t N, size_t K) {
     }
 }
 
+// One row of BM x 128 tiles, one workgroup per CU, with more column tiles than CUs: the tiles beyond the whole rounds
+// would run as a round of their own on a few CUs, so they are cut into K slices that fill the chip (M = 103,
+// N = 34304, K = 6656: 268 tiles, 133 us as two rounds against 89 us for hipBLASLt).  Worth its extra launch and
+// reduction (about 6 us) when the round it shortens is long: a round takes about half a microsecond per chunk
+// (M = 76, N = 39552, K = 640: 19.8 us as two rounds, 23.7 with the 53 tiles of the second in two slices).
+void one_row_tail(Plan &p, size_t bm, size_t stages, size_t N, size_t K, size_t cus, size_t partial_limit) {
+    const size_t tiles = div_ceil(N, (size_t)128), rem = tiles % cus;
+    const size_t tile_bytes = bm * 128 * sizeof(float);
+    if (tiles <= cus || rem == 0) return;
+    size_t ts = cus / rem < 16 ? cus / rem : 16;
+    while (ts >= 2 && (shortest_slice(K, 64, (int)ts) < 64 * stages || ts * rem * tile_bytes > partial_limit)) --ts;
+    if (ts >= 2 && (double)(K / 64) * (1.0 - 1.0 / (double)ts) > 12.0) {
+        p.tail_tiles = (int)rem;
+        p.tail_splits = (int)ts;
+        p.partial_bytes = ts * rem * tile_bytes;
+    }
+}
+
 }  // namespace
 
 bool skinny_supports(size_t M, size_t N, size_t K) {
@@ -491,24 +511,8 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
             }
             case KERNEL_MID128:
             case KERNEL_ROW64x128: {
-                // One workgroup per CU.  More column tiles than CUs: the tiles beyond the whole rounds would run as a
-                // round of their own on a few CUs, so they are cut into K slices that fill the chip (M = 103,
-                // N = 34304, K = 6656: 268 tiles, 133 us as two rounds against 89 us for hipBLASLt).
                 p.splits = 1;
-                const size_t tiles = div_ceil(N, (size_t)128), rem = tiles % cus;
-                const size_t tile_bytes = (size_t)(r.kernel == KERNEL_MID128 ? 128 : 64) * 128 * sizeof(float);
-                if (tiles > cus && rem > 0) {
-                    size_t ts = cus / rem < 16 ? cus / rem : 16;
-                    while (ts >= 2 && (shortest_slice(K, 64, (int)ts) < 64 * 5 || ts * rem * tile_bytes > limits.partial_bytes)) --ts;
-                    // worth its extra launch and reduction (about 6 us) when the round it shortens is long: a round
-                    // takes about half a microsecond per chunk (M = 76, N = 39552, K = 640: 19.8 us as two rounds, 23.7
-                    // with the 53 tiles of the second in two slices)
-                    if (ts >= 2 && (double)(K / 64) * (1.0 - 1.0 / (double)ts) > 12.0) {
-                        p.tail_tiles = (int)rem;
-                        p.tail_splits = (int)ts;
-                        p.partial_bytes = ts * rem * tile_bytes;
-                    }
-                }
+                one_row_tail(p, r.kernel == KERNEL_MID128 ? 128 : 64, 5, N, K, cus, limits.partial_bytes);
                 break;
             }
             default: {  // the split-K family: K slices across workgroups, then the ordered reduction
@@ -518,6 +522,21 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
             }
         }
         return p;
+    }
+    // M = 129 ... 192 against many columns: one row of 192x128 tiles, B copied non-temporally, where the last round of
+    // workgroups is at least 55 % full (N = 18432 ... 32768, 50688 ... 65536, ...).  Against the cost model's choice
+    // (192x192 tiles, 150 of them at N = 28672): N = 28672, K = 2048 ... 8192: 1.17 ... 1.30x (M = 192, K = 2048:
+    // 40.3 -> 31.4 us), K = 14336: 0.97 ... 1.12x; N = 57344: 1.01 ... 1.13x up to K = 8192, 0.96 ... 0.98x at 14336;
+    // N = 14336 (112 tiles): 0.81 ... 0.86x, N = 34304 (268 tiles): 0.76x.  The ring of four stages keeps three chunks
+    // of B in flight per CU where the 192x192 tile's three stages keep two.
+    {
+        const size_t tiles = div_ceil(N, (size_t)128), last = tiles % cus;
+        if (M > 128 && M <= 192 && N % 8 == 0 && K % 64 == 0 && K >= 2048 && K <= 12288 && tiles >= 144 &&
+            (last == 0 || last * 100 >= cus * 55)) {
+            p.kernel = KERNEL_ROW192x128;
+            p.splits = 1;
+            return p;
+        }
     }
     // Pipelined tiles: M and N may end inside a tile (guarded edges; the model charges whole
     // tiles), as long as rows of C stay 16-byte aligned and K is a whole number of chunks.
@@ -689,6 +708,7 @@ void run_plan(const Plan &p, const Workspace &ws, const void *A, const void *B, 
         case KERNEL_MID128: launch_pipelined_plan<Mid128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_MID128_S2: launch_pipelined<Mid128S2>(A, B, C, M, N, K, "hgemm_auto"); break;
         case KERNEL_ROW64x128: launch_pipelined_plan<Row64x128>(A, B, C, M, N, K, p, ws); break;
+        case KERNEL_ROW192x128: launch_pipelined_plan<Row192x128>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_SMALL64: launch_pipelined_plan<Small64>(A, B, C, M, N, K, p, ws); break;
         case KERNEL_SMALL64_W4: {
             const size_t chunks = K / 64 / (size_t)(p.splits > 1 ? p.splits : 1);
@@ -920,6 +940,7 @@ extern "C" const char *hgemm_kernel_name(int kernel) {
         case KERNEL_MID128: return "pipelined 128x128x64, 4 waves, 5-stage ring";
         case KERNEL_MID128_S2: return "pipelined 128x128x64, 4 waves, 2-stage ring";
         case KERNEL_ROW64x128: return "pipelined 64x128x64, 4 waves, 5-stage ring";
+        case KERNEL_ROW192x128: return "pipelined 192x128x64, 4 waves, 4-stage ring";
         case KERNEL_SMALL64: return "pipelined 64x64x64, 1 wave, 3-stage ring";
         case KERNEL_SMALL64_W4: return "tiled 64x64x64, 4 waves of 32x32, look-ahead ring";
         case KERNEL_T192: return "pipelined 192x192x64, 4 waves, 3-stage ring";

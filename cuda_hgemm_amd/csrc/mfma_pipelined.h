@@ -752,7 +752,7 @@ bool use_chained(PipeKernel which, size_t workgroups, size_t k_len) {
 // so only the tiles that run one row against many columns (128x128, 64x128; five stages) carry the second instantiation.
 template <class Cfg>
 constexpr bool stream_b_available() {
-    return Cfg::MI == 16 && Cfg::BN == 128 && (Cfg::BM == 128 || Cfg::BM == 64) && Cfg::STAGES == 5;
+    return Cfg::MI == 16 && Cfg::BN == 128 && (((Cfg::BM == 128 || Cfg::BM == 64) && Cfg::STAGES == 5) || (Cfg::BM == 192 && Cfg::STAGES == 4));
 }
 inline bool stream_b_pays(int tiles_m, size_t N, size_t K) { return tiles_m == 1 && N * K >= ((size_t)24 << 20); }
 

@@ -27,6 +27,7 @@ enum KernelId {
     KERNEL_PADDED,      // operands copied zero-padded to N % 8 == 0, K % 64 == 0, then the plan for that shape
     KERNEL_ROW64x128,   // pipelined 64x128x64, 4 waves side by side, 5-stage ring: one row of tiles for M <= 64 against many columns
     KERNEL_DECODE_RESIDENT,  // decode kernel for M <= 32 with A in registers: persistent workgroups walk over 16-column tiles; `splits` waves over K
+    KERNEL_ROW192x128,  // pipelined 192x128x64, 4 waves, 4-stage ring: one row of tiles for M = 129 ... 192 against many columns
 };
 
 struct Plan {

@@ -202,7 +202,7 @@ def test_auto_plan_invariants_over_many_shapes(hgemm_lib):
         s = p["splits"]
         assert s >= 1 and p["tail_splits"] >= 1, (m, n, k, p)
         if p["kernel"].startswith(("pipelined", "tiled", "split-K")):
-            shortest = {"pipelined 256x256": 2, "pipelined 192x192": 3, "pipelined 256x128": 3, "pipelined 128x128": 5,
+            shortest = {"pipelined 256x256": 2, "pipelined 192x192": 3, "pipelined 192x128": 4, "pipelined 256x128": 3, "pipelined 128x128": 5,
                         "pipelined 64x128": 5, "pipelined 64x64": 3, "tiled 64x64x64": 3, "split-K": 1}
             floor = [v for key, v in shortest.items() if p["kernel"].startswith(key)][0]
             if "2-stage ring" in p["kernel"]:

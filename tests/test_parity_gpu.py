@@ -507,6 +507,22 @@ def test_one_tile_row_with_more_tiles_than_cus(oracle, hgemm_lib, gpu, shape, ta
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
+@pytest.mark.parametrize("shape", [(192, 28672, 2048), (129, 18440, 4096), (160, 57344, 2112), (177, 20480, 8192)])
+def test_one_row_of_192x128_tiles(oracle, hgemm_lib, gpu, shape):
+    """M = 129 ... 192 against 144 column tiles or more: one row of 192x128 tiles on a four-stage ring, B copied
+    non-temporally; rows of the tile beyond M, a last column tile that ends inside N, more tiles than CUs."""
+    M, N, K = shape
+    plan = hgemm_lib.auto_plan(M, N, K)
+    assert plan["kernel"].startswith("pipelined 192x128x64, 4 waves, 4-stage") and plan["splits"] == 1 and plan["tail_tiles"] == 0, plan
+    A = oracle.fill((M, K), 45, 1, oracle.NORMAL, 0.0, 1.0)
+    B = oracle.fill((N, K), 45, 2, oracle.NORMAL, 0.0, 0.02)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    _assert_close(oracle, first, oracle.hgemm(A, B), K)
+    assert np.array_equal(first, second)
+    At, Bt = oracle.fill((M, K), 46, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 46, 2, oracle.TERNARY, 0, 1)
+    assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
+
+
 @pytest.mark.parametrize("M", [3, 17, 33, 100, 127])
 def test_skinny_ragged_M(oracle, hgemm_lib, gpu, M):
     N, K = 1024, 512
