@@ -319,14 +319,15 @@ double predict_subtile_us(const Candidate &big, const Candidate &small, size_t M
 // back) against B's (2 K bytes per column), counted twice.  The model's choice is 1.2 % behind the best count on
 // average (16 % at worst); the rule it replaces (the smallest power of two that divides K's chunks and gives three
 // quarters of the CUs a workgroup) was 22 % behind on average.  A slice is a whole number of 64-wide chunks, at least
-// two; slices differ by at most one chunk.
+// two (`min_chunks`: the pipelined tiles need as many as their ring has stages); slices differ by at most one chunk.
 // `slice_bytes`: fp32 partial sums of one slice; the slices together stay within `limit`.
-int choose_splits(size_t tiles, size_t M, size_t N, size_t cus, size_t K, size_t slice_bytes, size_t limit) {
+int choose_splits(size_t tiles, size_t M, size_t N, size_t cus, size_t K, size_t slice_bytes, size_t limit,
+                  size_t min_chunks = 2) {
     int best = 1;
     double best_us = 0.0;
     const double stream_us = 2.0 * (double)N * (double)K / 5e6;
     for (int s = 1; s <= 16; ++s) {
-        if (s > 1 && (K % 64 != 0 || K / 64 / (size_t)s < 2 || (size_t)s * slice_bytes > limit)) break;
+        if (s > 1 && (K % 64 != 0 || K / 64 / (size_t)s < min_chunks || (size_t)s * slice_bytes > limit)) break;
         const size_t wgs = tiles * (size_t)s;
         const double balance = (double)wgs / (double)(div_ceil(wgs, cus) * cus);
         const double partials = s > 1 ? 8.0 * s * (double)M / (double)K : 0.0;
@@ -425,6 +426,12 @@ constexpr SmallMRule SMALL_M_RULES[] = {
     // K = 4096, 8192 x N = 18432 ... 57344: 0.97 ... 1.27x over the split-K 32x64 kernel; at K <= 2048 that kernel stays
     // ahead against N >= 28672 (0.92 ... 0.98x).
     {17, 32, 18432, ANY, 4096, ANY, 0, ANY, 0, KERNEL_ROW64x128},
+    // M = 33 ... 128 against N = 6144 ... 18431 with a long K: the same two tiles with K in slices (their copies of B
+    // non-temporal too), the slice count by the split-K family's model: over N = 6144 ... 16384, M = 64 and 128,
+    // K = 8192 and 16384: 0.99 ... 1.34x of the split-K kernels at their best slice count (median 1.17x; M = 128,
+    // N = 10240, K = 16384: 106.9 -> 79.8 us); at K = 4096 mixed (0.92 ... 1.13x), at K = 2048 behind (0.80 ... 1.07x).
+    {65, 128, 6144, ANY, 8192, ANY, 0, ANY, 0, KERNEL_MID128},
+    {33, 64, 6144, ANY, 8192, ANY, 0, ANY, 0, KERNEL_ROW64x128},
     // --- everything else with N % 64 == 0 and K % 64 == 0: the split-K family, the tile by M; 128-wide tiles where
     // N gives enough of them and is a multiple of 128 (they stream B better).
     {1, 32, 1, ANY, 1, ANY, 0, ANY, 0, KERNEL_SPLIT_32x64},
@@ -511,8 +518,14 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
             }
             case KERNEL_MID128:
             case KERNEL_ROW64x128: {
-                p.splits = 1;
-                one_row_tail(p, r.kernel == KERNEL_MID128 ? 128 : 64, 5, N, K, cus, limits.partial_bytes);
+                // up to one workgroup per CU: K slices by the split-K family's model (the same balance against the
+                // same partial sums); more tiles than CUs: whole rounds unsliced, the rest in K slices
+                const size_t tiles = div_ceil(N, (size_t)128);
+                // (from K = 8192: below, slices were measured level or behind -- M = 96, N = 18432, K = 4096: 40.8 us
+                // unsliced, 43.6 in three)
+                p.splits = tiles <= cus && K >= 8192 ? choose_splits(tiles, M, N, cus, K, slice_bytes, limits.partial_bytes, 5) : 1;
+                if (p.splits > 1) p.partial_bytes = (size_t)p.splits * slice_bytes;
+                if (tiles > cus) one_row_tail(p, r.kernel == KERNEL_MID128 ? 128 : 64, 5, N, K, cus, limits.partial_bytes);
                 break;
             }
             default: {  // the split-K family: K slices across workgroups, then the ordered reduction

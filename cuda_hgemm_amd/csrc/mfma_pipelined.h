@@ -771,7 +771,7 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
             HGEMM_CHECK_HIP_ERROR(
                 hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_chained_kernel<Cfg, SPLIT, EDGE>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
-        if constexpr (stream_b_available<Cfg>() && !SPLIT)
+        if constexpr (stream_b_available<Cfg>())
             HGEMM_CHECK_HIP_ERROR(
                 hipFuncSetAttribute(reinterpret_cast<const void *>(&hgemm_pipelined_kernel<Cfg, SPLIT, EDGE, true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
@@ -782,11 +782,11 @@ void launch_pipelined_impl(const void *A, const void *B, void *C, float *partial
     if (blocks < 0) blocks = tiles_m * tiles_n - first_block;
     HGEMM_CHECK(first_block >= 0 && blocks >= 1 && first_block + blocks <= tiles_m * tiles_n);
     HGEMM_CHECK(splits >= 1 && (SPLIT || splits == 1) && (size_t)blocks * (size_t)splits < ((size_t)1 << 31));
-    if constexpr (stream_b_available<Cfg>() && !SPLIT) {
+    if constexpr (stream_b_available<Cfg>()) {
         if (which != PipeKernel::Chained && stream_b_pays(tiles_m, N, K)) {
-            hgemm_pipelined_kernel<Cfg, SPLIT, EDGE, true><<<dim3(blocks), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
+            hgemm_pipelined_kernel<Cfg, SPLIT, EDGE, true><<<dim3(blocks * splits), dim3(Cfg::THREADS), Cfg::LDS_BYTES, nullptr>>>(
                 reinterpret_cast<const half_t *>(A), reinterpret_cast<const half_t *>(B), reinterpret_cast<half_t *>(C),
-                partial, (int)M, (int)N, (int)K, 1, tiles_m, tiles_n, first_block, tail_tiles, subdiv);
+                partial, (int)M, (int)N, (int)K, splits, tiles_m, tiles_n, first_block, tail_tiles, subdiv);
             HGEMM_CHECK_HIP_ERROR(hipGetLastError());
             return;
         }

@@ -469,7 +469,7 @@ def test_small_m_against_a_large_b(oracle, hgemm_lib, gpu, shape):
 @pytest.mark.parametrize("shape", [(128, 28672, 4096), (100, 18440, 1024), (65, 20480, 2048), (128, 18432, 1088),
                                    (97, 24584, 1024), (128, 28672, 320 + 704),
                                    (64, 28672, 4096), (33, 18440, 1024), (50, 20480, 2048), (64, 24584, 1088), (64, 28672, 320),
-                                   (128, 28672, 384), (25, 28672, 4096), (32, 18432, 8192)])
+                                   (128, 28672, 384), (25, 28672, 4096), (32, 18432, 4096)])
 def test_one_tile_row_against_many_column_tiles(oracle, hgemm_lib, gpu, shape):
     """M = 33 ... 128 against N >= 18432: one launch of the pipelined kernel on a 128x128 tile (a 64x128 tile up to
     M = 64) whose copies of B carry the non-temporal hint (from 48 MB of B on; the smaller cases run the same rule
@@ -484,6 +484,24 @@ def test_one_tile_row_against_many_column_tiles(oracle, hgemm_lib, gpu, shape):
     _assert_close(oracle, first, oracle.hgemm(A, B), K)
     assert np.array_equal(first, second)
     At, Bt = oracle.fill((M, K), 42, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 42, 2, oracle.TERNARY, 0, 1)
+    assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
+
+
+@pytest.mark.parametrize("shape,slices", [((128, 6144, 8192), 5), ((64, 8192, 8192), 4), ((100, 12296, 8256), 5),
+                                           ((40, 18432, 12352), 7), ((32, 18432, 8192), 5), ((128, 16384, 8192), 2)])
+def test_one_tile_row_in_k_slices(oracle, hgemm_lib, gpu, shape, slices):
+    """M = 17 ... 128 with a long K against fewer column tiles than CUs: the one-row 128x128 / 64x128 tiles with K in
+    slices (B copied non-temporally in the sliced launch as well), slice counts that do and do not divide K's chunks,
+    a last column tile that ends inside N."""
+    M, N, K = shape
+    plan = hgemm_lib.auto_plan(M, N, K)
+    assert plan["kernel"].startswith("pipelined %s" % ("128x128x64" if M > 64 else "64x128x64")) and plan["splits"] == slices, plan
+    A = oracle.fill((M, K), 47, 1, oracle.NORMAL, 0.0, 1.0)
+    B = oracle.fill((N, K), 47, 2, oracle.NORMAL, 0.0, 0.02)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    _assert_close(oracle, first, oracle.hgemm(A, B), K)
+    assert np.array_equal(first, second)
+    At, Bt = oracle.fill((M, K), 48, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 48, 2, oracle.TERNARY, 0, 1)
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
