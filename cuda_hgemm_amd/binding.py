@@ -50,6 +50,7 @@ HELPER_SYMBOLS = [
     "hgemm_tflops", "hgemm_bytes", "hgemm_version",
     "hgemm_reserve_workspace", "hgemm_release_workspace", "hgemm_auto_workspace_bytes",
     "hgemm_auto_static_workspace", "hgemm_static_workspace_bytes",
+    "hgemm_auto_tune", "hgemm_auto_tune_plans", "hgemm_auto_forget_tuning", "hgemm_auto_plan_is_tuned",
 ]
 
 
@@ -115,6 +116,12 @@ class HgemmLibrary:
         d.hgemm_auto_plan_tail_kernel.argtypes, d.hgemm_auto_plan_tail_kernel.restype = [_SZ, _SZ, _SZ], C.c_int
         d.hgemm_auto_plan_chained.argtypes, d.hgemm_auto_plan_chained.restype = [_SZ, _SZ, _SZ], C.c_int
         d.hgemm_kernel_name.argtypes, d.hgemm_kernel_name.restype = [C.c_int], C.c_char_p
+        d.hgemm_auto_tune.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, _SZ, _SZ, _SZ, C.c_int, C.c_int]
+        d.hgemm_auto_tune.restype = C.c_int
+        d.hgemm_auto_tune_plans.argtypes = [_SZ, _SZ, _SZ, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        d.hgemm_auto_tune_plans.restype = C.c_int
+        d.hgemm_auto_forget_tuning.argtypes, d.hgemm_auto_forget_tuning.restype = [], None
+        d.hgemm_auto_plan_is_tuned.argtypes, d.hgemm_auto_plan_is_tuned.restype = [_SZ, _SZ, _SZ], C.c_int
         d.hgemm_small_m_rule.argtypes = [C.c_int, C.POINTER(_SZ), C.POINTER(C.c_int)]
         d.hgemm_small_m_rule.restype = C.c_int
         d.hgemm_variant_count.argtypes, d.hgemm_variant_count.restype = [], C.c_int
@@ -170,6 +177,26 @@ class HgemmLibrary:
                 "chained": bool(self.dll.hgemm_auto_plan_chained(M, N, K)),
                 "tail_tiles": tail_tiles, "tail_splits": tail_splits.value,
                 "tail_kernel": self.dll.hgemm_kernel_name(self.dll.hgemm_auto_plan_tail_kernel(M, N, K)).decode()}
+
+    def tune(self, A, B, C_out, M: int, N: int, K: int, max_plans: int = 6, cold: bool = False) -> int:
+        """Times up to ``max_plans`` plans for the shape on these operands and keeps the fastest for every later
+        ``hgemm_auto`` call of the shape (``hgemm_auto_tune``); ``cold``: with the caches flushed before every timed
+        launch.  Returns how many were timed."""
+        return self.dll.hgemm_auto_tune(_tensor_ptr(A, M, K, "A"), _tensor_ptr(B, N, K, "B (stored as N rows of K)"),
+                                        _tensor_ptr(C_out, M, N, "C"), M, N, K, max_plans, 1 if cold else 0)
+
+    def tune_plans(self, M: int, N: int, K: int, max_plans: int = 6) -> List[dict]:
+        """What ``tune`` would time, best first by the model (no launch)."""
+        kernels, splits = (C.c_int * max_plans)(), (C.c_int * max_plans)()
+        n = self.dll.hgemm_auto_tune_plans(M, N, K, max_plans, kernels, splits)
+        return [{"kernel_id": kernels[i], "kernel": self.dll.hgemm_kernel_name(kernels[i]).decode(), "splits": splits[i]}
+                for i in range(n)]
+
+    def forget_tuning(self) -> None:
+        self.dll.hgemm_auto_forget_tuning()
+
+    def plan_is_tuned(self, M: int, N: int, K: int) -> bool:
+        return bool(self.dll.hgemm_auto_plan_is_tuned(M, N, K))
 
     def small_m_rules(self) -> List[dict]:
         """The table behind hgemm_auto's choice for M <= 128, in order (first covering row wins)."""

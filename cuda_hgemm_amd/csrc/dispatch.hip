@@ -8,6 +8,8 @@
 #include "mfma_skinny.h"
 #include "plan.h"
 
+#include <atomic>
+#include <map>
 #include <mutex>
 
 namespace hgemm {
@@ -468,16 +470,17 @@ bool small_m_kernel_supports(int kernel, size_t M, size_t N, size_t K) {
 
 // One row of BM x 128 tiles, one workgroup per CU, with more column tiles than CUs: the tiles beyond the whole rounds
 // would run as a round of their own on a few CUs, so they are cut into K slices that fill the chip (M = 103,
-// N = 34304, K = 6656: 268 tiles, 133 us as two rounds against 89 us for hipBLASLt).  Worth its extra launch and
-// reduction (about 6 us) when the round it shortens is long: a round takes about half a microsecond per chunk
-// (M = 76, N = 39552, K = 640: 19.8 us as two rounds, 23.7 with the 53 tiles of the second in two slices).
+// N = 34304, K = 6656: 268 tiles, 133 us as two rounds, 80 us this way; hipBLASLt 89 us).  Worth its extra launch and
+// reduction when the round it shortens is long, i.e. from K of about 2500 ... 4000 on (M = 76, N = 39552, K = 640:
+// 19.8 us as two rounds, 23.7 with the 53 tiles of the second in two slices; K = 1280 ... 1792 with the tail: 78 ... 81 %
+// of hipBLASLt, K = 4352 ... 6656: 86 ... 111 %).
 void one_row_tail(Plan &p, size_t bm, size_t stages, size_t N, size_t K, size_t cus, size_t partial_limit) {
     const size_t tiles = div_ceil(N, (size_t)128), rem = tiles % cus;
     const size_t tile_bytes = bm * 128 * sizeof(float);
     if (tiles <= cus || rem == 0) return;
     size_t ts = cus / rem < 16 ? cus / rem : 16;
     while (ts >= 2 && (shortest_slice(K, 64, (int)ts) < 64 * stages || ts * rem * tile_bytes > partial_limit)) --ts;
-    if (ts >= 2 && (double)(K / 64) * (1.0 - 1.0 / (double)ts) > 12.0) {
+    if (ts >= 2 && (double)(K / 64) * (1.0 - 1.0 / (double)ts) > 32.0) {
         p.tail_tiles = (int)rem;
         p.tail_splits = (int)ts;
         p.partial_bytes = ts * rem * tile_bytes;
@@ -490,6 +493,22 @@ bool skinny_supports(size_t M, size_t N, size_t K) {
     return M >= 1 && M <= 128 && N > 0 && N % 64 == 0 && K > 0 && K % 64 == 0;
 }
 
+bool same_choice(const Plan &a, const Plan &b) {
+    return a.kernel == b.kernel && a.splits == b.splits && a.tail_tiles == b.tail_tiles && a.tail_splits == b.tail_splits &&
+           a.tail_kernel == b.tail_kernel;
+}
+bool left_out(const PlanLimits &limits, const Plan &p) {
+    for (int i = 0; i < limits.excluded_count; ++i)
+        if (same_choice(limits.excluded[i], p)) return true;
+    return false;
+}
+bool left_out(const PlanLimits &limits, int kernel, int splits, int tail_tiles = 0, int tail_splits = 1,
+              int tail_kernel = KERNEL_NONE) {
+    Plan p;
+    p.kernel = kernel, p.splits = splits, p.tail_tiles = tail_tiles, p.tail_splits = tail_splits, p.tail_kernel = tail_kernel;
+    return left_out(limits, p);
+}
+
 // M <= 128: choices come from timing every candidate (tile x slices) on the specification's
 // decode shapes on an MI355X, operands rotated so small problems read HBM.  Larger,
 // tile-aligned shapes: the cheapest (tile, slices) pair under the cost model above.
@@ -500,7 +519,10 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     const size_t slice_bytes = M * N * sizeof(float);  // fp32 partial sums of one K slice of the whole product
     // M <= 128: the first row of the table above that covers the shape and whose kernel can run it
     for (const SmallMRule &r : SMALL_M_RULES) {
-        if (!small_m_rule_covers(r, M, N, K) || !small_m_kernel_supports(r.kernel, M, N, K)) continue;
+        if (M > 128) break;
+        if (limits.every_small_m_kernel ? (M < (size_t)r.m_lo || M > (size_t)r.m_hi) : !small_m_rule_covers(r, M, N, K)) continue;
+        if (!small_m_kernel_supports(r.kernel, M, N, K)) continue;
+        p = Plan();
         p.kernel = r.kernel;
         switch (r.kernel) {
             case KERNEL_DECODE_RING: p.splits = decode_ring_waves(M, N, K, cus); break;
@@ -534,8 +556,10 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
                 if (p.splits > 1) p.partial_bytes = (size_t)p.splits * slice_bytes;
             }
         }
+        if (left_out(limits, p)) continue;
         return p;
     }
+    p = Plan();
     // M = 129 ... 192 against many columns: one row of 192x128 tiles, B copied non-temporally, where the last round of
     // workgroups is at least 55 % full (N = 18432 ... 32768, 50688 ... 65536, ...).  Against the cost model's choice
     // (192x192 tiles, 150 of them at N = 28672): N = 28672, K = 2048 ... 8192: 1.17 ... 1.30x (M = 192, K = 2048:
@@ -545,7 +569,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
     {
         const size_t tiles = div_ceil(N, (size_t)128), last = tiles % cus;
         if (M > 128 && M <= 192 && N % 8 == 0 && K % 64 == 0 && K >= 2048 && K <= 12288 && tiles >= 144 &&
-            (last == 0 || last * 100 >= cus * 55)) {
+            (last == 0 || last * 100 >= cus * 55) && !left_out(limits, KERNEL_ROW192x128, 1)) {
             p.kernel = KERNEL_ROW192x128;
             p.splits = 1;
             return p;
@@ -570,6 +594,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
             if (c.kernel == KERNEL_SMALL64 && M % 64 == 0 && N % 64 == 0 && (M / 64) * (N / 64) * (size_t)s <= cus) continue;
             if (K % 64 || shortest_slice(K, 64, s) < (size_t)64 * c.stages) break;
             if (s > 1 && (size_t)s * slice_bytes > limits.partial_bytes) break;
+            if (left_out(limits, c.kernel, s)) continue;
             const double t = predict_us(c, M, N, K, s, cus);
             if (p.kernel == KERNEL_NONE || t < best) {
                 best = t;
@@ -589,6 +614,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
             for (int ts = 2; ts <= 16; ++ts) {
                 if (K % 64 || shortest_slice(K, 64, ts) < (size_t)64 * c.stages || rem * ts > slots) break;
                 if ((size_t)ts * rem * c.bm * c.bn * sizeof(float) > limits.partial_bytes) break;
+                if (left_out(limits, c.kernel, 1, (int)rem, ts)) continue;
                 const double t = predict_tail_us(c, M, N, K, ts, cus);
                 if (p.kernel != KERNEL_NONE && t < best) {
                     best = t;
@@ -606,7 +632,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
                     if (small.kernel == KERNEL_BIG256 || small.kernel == KERNEL_SMALL64_W4 || small.kernel == KERNEL_MID128_S2 ||
                         c.bm % small.bm || c.bn % small.bn)
                         continue;
-                    if (K < (size_t)64 * small.stages) continue;
+                    if (K < (size_t)64 * small.stages || left_out(limits, c.kernel, 1, (int)rem, 1, small.kernel)) continue;
                     const double t = predict_subtile_us(c, small, M, N, K, cus);
                     if (p.kernel != KERNEL_NONE && t < best) {
                         best = t;
@@ -623,6 +649,7 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
         }
     }
     if (p.kernel != KERNEL_NONE) return p;
+    if (limits.excluded_count > 0) return Plan();  // the tuner's question has no further answer
     if (N % 64 == 0 && K % 64 == 0) {  // any M: rows beyond M are guarded
         p.kernel = KERNEL_SPLIT_64x64;
         p.splits = choose_splits(div_ceil(M, 64) * (N / 64), M, N, cus, K, slice_bytes, limits.partial_bytes);
@@ -782,14 +809,46 @@ struct CachedPlan {
 };
 constexpr int PLAN_CACHE_SLOTS = 64;
 
+// Plans that hgemm_auto_tune measured to be the fastest for a shape: process-wide, consulted before the model.  The
+// per-thread tables below are thrown away whenever this one changes (`g_tuned_version`).
+struct TunedShape {
+    size_t M, N, K;
+    bool operator<(const TunedShape &o) const { return M != o.M ? M < o.M : N != o.N ? N < o.N : K < o.K; }
+};
+std::map<TunedShape, Plan> g_tuned;
+std::mutex g_tuned_mutex;
+std::atomic<unsigned> g_tuned_version{0};
+
+bool tuned_plan(size_t M, size_t N, size_t K, Plan *out) {
+    if (g_tuned_version.load(std::memory_order_acquire) == 0) return false;  // nothing was ever tuned: no lock
+    std::lock_guard<std::mutex> lock(g_tuned_mutex);
+    const auto it = g_tuned.find(TunedShape{M, N, K});
+    if (it == g_tuned.end()) return false;
+    *out = it->second;
+    return true;
+}
+
+// the plan hgemm_auto runs and the hgemm_auto_plan* queries report: the tuned one if there is one, else the model's
+Plan current_plan(size_t M, size_t N, size_t K) {
+    Plan p;
+    return tuned_plan(M, N, K, &p) ? p : plan_for(M, N, K);
+}
+
 const Plan &cached_plan(size_t M, size_t N, size_t K, bool without_workspace = false) {
     static thread_local CachedPlan cache[2][PLAN_CACHE_SLOTS];
+    static thread_local unsigned seen_version = 0;
+    const unsigned version = g_tuned_version.load(std::memory_order_acquire);
+    if (version != seen_version) {
+        for (auto &table : cache)
+            for (CachedPlan &slot : table) slot = CachedPlan();
+        seen_version = version;
+    }
     const size_t h = (M * 0x9e3779b97f4a7c15ull) ^ (N * 0xc2b2ae3d27d4eb4full) ^ (K * 0x165667b19e3779f9ull);
     CachedPlan &slot = cache[without_workspace ? 1 : 0][(h >> 32) % PLAN_CACHE_SLOTS];
     if (slot.M != M || slot.N != N || slot.K != K) {
         PlanLimits limits;
         if (without_workspace) limits.partial_bytes = limits.operand_bytes = 0;
-        slot.plan = plan_for(M, N, K, limits);
+        if (without_workspace || !tuned_plan(M, N, K, &slot.plan)) slot.plan = plan_for(M, N, K, limits);
         slot.M = M, slot.N = N, slot.K = K;
     }
     return slot.plan;
@@ -828,6 +887,120 @@ extern "C" int hgemm_skinny_supports(size_t M, size_t N, size_t K) { return skin
 extern "C" void hgemm_auto(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K) {
     check_operands(A, B, C, M, N, K);
     run_with_heap_workspace(A, B, C, M, N, K);
+}
+
+// The plans hgemm_auto_tune times for a shape, best first by the model: the plan hgemm_auto runs anyway, then the
+// best that is none of the earlier.
+constexpr int TUNE_MOST_PLANS = 12;
+int plans_to_time(size_t M, size_t N, size_t K, int max_plans, Plan *plans) {
+    if (max_plans < 1) max_plans = 1;
+    if (max_plans > TUNE_MOST_PLANS) max_plans = TUNE_MOST_PLANS;
+    int count = 0;
+    PlanLimits limits;
+    limits.excluded = plans;
+    while (count < max_plans) {
+        limits.excluded_count = count;
+        limits.every_small_m_kernel = count > 0;
+        const Plan p = plan_for(M, N, K, limits);
+        if (p.kernel == KERNEL_NONE) break;
+        plans[count++] = p;
+        if (p.kernel == KERNEL_PADDED || p.kernel == KERNEL_RAGGED || p.kernel == KERNEL_SIMT) break;  // nothing to choose from
+    }
+    return count;
+}
+
+// What hgemm_auto_tune would time, without launching anything: kernel ids and K slices of up to max_plans plans.
+extern "C" int hgemm_auto_tune_plans(size_t M, size_t N, size_t K, int max_plans, int *kernels, int *splits) {
+    Plan plans[TUNE_MOST_PLANS];
+    const int count = plans_to_time(M, N, K, max_plans, plans);
+    for (int i = 0; i < count; ++i) {
+        if (kernels) kernels[i] = plans[i].kernel;
+        if (splits) splits[i] = plans[i].splits;
+    }
+    return count;
+}
+
+// Streams over a buffer larger than the caches hold, so that what was cached before is not afterwards.
+__global__ void __launch_bounds__(256) cache_flush_kernel(floatx4 *buffer, size_t count, float value) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride)
+        buffer[i] = floatx4{value, value, value, value};
+}
+
+// Times the model's best plans for this shape on the caller's operands and keeps the fastest for every later
+// hgemm_auto call of the shape in this process: the first plan is the one hgemm_auto would run anyway, each next
+// one the best that is none of the earlier (another tile, another slice count, for M <= 128 another kernel).  One
+// untimed and three timed launches per plan, each timed launch bracketed by events on the null stream; with
+// HGEMM_TUNE_COLD 512 MiB are streamed through the device before each timed launch, so that A and B come from HBM as
+// they do for a caller whose weights do not stay cached between calls.  The call returns when the device is idle
+// and C holds the product as the kept plan computes it.
+extern "C" int hgemm_auto_tune(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K,
+                               int max_plans, int flags) {
+    check_operands(A, B, C, M, N, K);
+    Plan plans[TUNE_MOST_PLANS];
+    const int count = plans_to_time(M, N, K, max_plans, plans);
+    constexpr size_t FLUSH_BYTES = (size_t)512 << 20;
+    floatx4 *flush = nullptr;
+    if ((flags & HGEMM_TUNE_COLD) && hipMalloc(reinterpret_cast<void **>(&flush), FLUSH_BYTES) != hipSuccess) {
+        (void)hipGetLastError();
+        flush = nullptr;  // no memory for it: the plans are timed on whatever the caches hold
+    }
+    hipEvent_t start, stop;
+    HGEMM_CHECK_HIP_ERROR(hipEventCreate(&start));
+    HGEMM_CHECK_HIP_ERROR(hipEventCreate(&stop));
+    int best = -1, timed = 0;
+    float best_ms = 0.0f;
+    auto run = [&](const Plan &p) {  // false: the workspace the plan needs could not be had
+        std::lock_guard<std::mutex> lock(g_heap_mutex);
+        Workspace ws;
+        if ((p.partial_bytes || p.operand_bytes) && !heap_workspace(p.partial_bytes, p.operand_bytes, &ws, false)) return false;
+        run_plan(p, ws, A, B, C, M, N, K);
+        return true;
+    };
+    for (int i = 0; i < count; ++i) {
+        if (!run(plans[i])) continue;
+        float total_ms = 0.0f;
+        for (int launch = 0; launch < 3; ++launch) {
+            if (flush) {
+                cache_flush_kernel<<<dim3(2048), dim3(256), 0, nullptr>>>(flush, FLUSH_BYTES / sizeof(floatx4), (float)launch);
+                HGEMM_CHECK_HIP_ERROR(hipGetLastError());
+            }
+            HGEMM_CHECK_HIP_ERROR(hipEventRecord(start, nullptr));
+            run(plans[i]);
+            HGEMM_CHECK_HIP_ERROR(hipEventRecord(stop, nullptr));
+            HGEMM_CHECK_HIP_ERROR(hipEventSynchronize(stop));
+            float ms = 0.0f;
+            HGEMM_CHECK_HIP_ERROR(hipEventElapsedTime(&ms, start, stop));
+            total_ms += ms;
+        }
+        ++timed;
+        if (best < 0 || total_ms < best_ms) best = i, best_ms = total_ms;
+    }
+    HGEMM_CHECK_HIP_ERROR(hipEventDestroy(start));
+    HGEMM_CHECK_HIP_ERROR(hipEventDestroy(stop));
+    HGEMM_CHECK_MSG(best >= 0, "hgemm_auto_tune: no plan for M=%zu N=%zu K=%zu could be run", M, N, K);
+    {
+        std::lock_guard<std::mutex> lock(g_tuned_mutex);
+        g_tuned[TunedShape{M, N, K}] = plans[best];
+        g_tuned_version.fetch_add(1, std::memory_order_release);
+    }
+    run(plans[best]);
+    HGEMM_CHECK_HIP_ERROR(hipDeviceSynchronize());
+    if (flush) HGEMM_CHECK_HIP_ERROR(hipFree(flush));
+    return timed;
+}
+
+// Forgets every tuned plan: hgemm_auto goes by the model again.
+extern "C" void hgemm_auto_forget_tuning(void) {
+    std::lock_guard<std::mutex> lock(g_tuned_mutex);
+    g_tuned.clear();
+    g_tuned_version.fetch_add(1, std::memory_order_release);
+}
+
+// 1 if the shape's plan was set by hgemm_auto_tune.
+extern "C" int hgemm_auto_plan_is_tuned(size_t M, size_t N, size_t K) {
+    Plan p;
+    return tuned_plan(M, N, K, &p) ? 1 : 0;
 }
 
 // The tuned kernel by tile, as entry points of their own.  M and N may end inside a tile.
@@ -898,7 +1071,7 @@ extern "C" int hgemm_auto_static_workspace(const hgemm_half *A, const hgemm_half
 extern "C" size_t hgemm_static_workspace_bytes(void) { return STATIC_WORKSPACE_BYTES; }
 
 extern "C" size_t hgemm_auto_workspace_bytes(size_t M, size_t N, size_t K, size_t *operand_bytes) {
-    const Plan p = plan_for(M, N, K);
+    const Plan p = current_plan(M, N, K);
     if (operand_bytes) *operand_bytes = p.operand_bytes;
     return p.partial_bytes;
 }
@@ -906,14 +1079,14 @@ extern "C" int hgemm_auto_supports(size_t M, size_t N, size_t K) { return M > 0 
 
 // Which kernel and how many K slices hgemm_auto uses for a shape (for reports and tests).
 extern "C" int hgemm_auto_plan(size_t M, size_t N, size_t K, int *splits) {
-    const Plan p = plan_for(M, N, K);
+    const Plan p = current_plan(M, N, K);
     if (splits) *splits = p.splits;
     return p.kernel;
 }
 // How hgemm_auto treats the last, partly filled round of a large grid: the number of
 // workgroups in it that run in K slices (0: none) and, through `splits`, the slice count.
 extern "C" int hgemm_auto_plan_tail(size_t M, size_t N, size_t K, int *splits) {
-    const Plan p = plan_for(M, N, K);
+    const Plan p = current_plan(M, N, K);
     if (splits) *splits = p.tail_splits;
     return p.tail_tiles;
 }
@@ -931,10 +1104,10 @@ extern "C" int hgemm_small_m_rule(int index, size_t *bounds, int *flags) {
     return r.kernel;
 }
 // Kernel id of the smaller tile that takes over the last round (0: none).
-extern "C" int hgemm_auto_plan_tail_kernel(size_t M, size_t N, size_t K) { return plan_for(M, N, K).tail_kernel; }
+extern "C" int hgemm_auto_plan_tail_kernel(size_t M, size_t N, size_t K) { return current_plan(M, N, K).tail_kernel; }
 // 1 if the plan's main launch runs the chained kernel of its tile, 0 for the interleaved one.
 extern "C" int hgemm_auto_plan_chained(size_t M, size_t N, size_t K) {
-    const Plan p = plan_for(M, N, K);
+    const Plan p = current_plan(M, N, K);
     if (p.splits < 1) return 0;
     const size_t k_len = shortest_slice(K, 64, p.splits);
     auto workgroups = [&](size_t bm, size_t bn) {  // of the main launch

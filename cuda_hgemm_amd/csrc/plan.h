@@ -54,6 +54,12 @@ struct Workspace {
 struct PlanLimits {
     size_t partial_bytes = 512ull << 20;
     size_t operand_bytes = 1024ull << 20;
+    // For the tuner, which asks for the best plan, then the best plan that is none of those it already has, and so
+    // on: plans to leave out (compared by kernel, K slices and the treatment of the last round), and whether the
+    // small-M table's rows apply to every shape their kernel can run rather than to their boxes only.
+    const Plan *excluded = nullptr;
+    int excluded_count = 0;
+    bool every_small_m_kernel = false;
 };
 
 bool skinny_supports(size_t M, size_t N, size_t K);

@@ -135,6 +135,26 @@ int hgemm_auto_plan_tail_kernel(size_t M, size_t N, size_t K);
  * interleaved one (hgemm_mfma_pipelined_*) or a kernel of another family. */
 int hgemm_auto_plan_chained(size_t M, size_t N, size_t K);
 const char *hgemm_kernel_name(int kernel);
+/* Tuning on the caller's operands, for callers who run a shape many times: times up to max_plans (at most 12)
+ * plans for the shape -- the one hgemm_auto would run, then the cost model's next best, each different in tile,
+ * K slices or, for M <= 128, kernel -- with one untimed and three timed launches each (`flags`: 0 or
+ * HGEMM_TUNE_COLD), and keeps the fastest for
+ * every later hgemm_auto call of this shape in this process, from any thread; the hgemm_auto_plan* queries then
+ * report the kept plan.  Blocks until the device is idle; C holds the product as the kept plan computes it (every
+ * plan computes the same product; plans that slice K differently differ in the last bit of some outputs).  May
+ * allocate the workspace.  Returns the number of plans timed.  The vendor comparator is tuned the same way at its
+ * first call of a shape (include/hgemm_hipblaslt.h).  No counterpart in the reference, whose kernels are one per
+ * entry point. */
+#define HGEMM_TUNE_COLD 1 /* flags: stream 512 MiB through the device before every timed launch, so that A and B come
+                           * from HBM -- for callers whose operands (weights) do not stay cached between calls */
+int hgemm_auto_tune(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K,
+                    int max_plans, int flags);
+/* The plans hgemm_auto_tune would time, best first by the model, without a launch: kernel ids (for
+ * hgemm_kernel_name) and K slices into arrays of max_plans entries (either may be NULL); returns their number. */
+int hgemm_auto_tune_plans(size_t M, size_t N, size_t K, int max_plans, int *kernels, int *splits);
+/* Forgets every kept plan; 1 if the shape has one. */
+void hgemm_auto_forget_tuning(void);
+int hgemm_auto_plan_is_tuned(size_t M, size_t N, size_t K);
 /* The table behind hgemm_auto's choice for M <= 128 (decode-shaped products), row by row: the
  * first row that covers a shape, and whose kernel can run it, decides.  bounds receives
  * {m_lo, m_hi, n_lo, n_hi, k_lo, k_hi, b_lo, b_hi}, all inclusive, b = N * K (elements of B);

@@ -137,3 +137,41 @@ def test_device_buffers_without_torch(oracle, hgemm_lib, gpu):
         buf.free()
     with pytest.raises(ValueError):
         hgemm_lib.call("hgemm_auto", Ad, Bd, Cd, M, N, K)
+
+
+@pytest.mark.parametrize("shape", [(384, 6144, 5120), (64, 4096, 4096), (16, 28672, 4096), (1000, 4000, 4096),
+                                   (100, 100, 100)])
+def test_tuning_on_the_callers_operands(oracle, hgemm_lib, gpu, shape):
+    """hgemm_auto_tune times the model's best plans for a shape and keeps the fastest: the kept plan is one of those
+    hgemm_auto_tune_plans lists, the plan queries report it, C holds its product (within the tolerance of the
+    specification: plans that slice K differently differ in the last bit), hgemm_auto then reproduces C bit for bit,
+    and forgetting the tuning brings the model's plan back.  A shape with nothing to choose from (no tile divides
+    it) times one plan."""
+    import torch
+    M, N, K = shape
+    hgemm_lib.forget_tuning()
+    model_plan = hgemm_lib.auto_plan(M, N, K)
+    listed = hgemm_lib.tune_plans(M, N, K, 6)
+    assert 1 <= len(listed) <= 6 and listed[0]["kernel_id"] == model_plan["kernel_id"] and listed[0]["splits"] == model_plan["splits"]
+    A = oracle.fill((M, K), 91, 1, oracle.NORMAL, 0.0, 1.0)
+    B = oracle.fill((N, K), 91, 2, oracle.NORMAL, 0.0, 0.02)
+    Ad, Bd = _to_gpu(A, gpu), _to_gpu(B, gpu)
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=gpu)
+    try:
+        print(f"[gpu] hgemm_auto_tune M={M} N={N} K={K}", flush=True)
+        timed = hgemm_lib.tune(Ad, Bd, C, M, N, K, 6, cold=(M % 2 == 0 and N == 4096))
+        assert 1 <= timed <= len(listed) and hgemm_lib.plan_is_tuned(M, N, K)
+        if shape == (100, 100, 100):
+            assert timed == 1
+        kept = hgemm_lib.auto_plan(M, N, K)
+        assert any(kept["kernel_id"] == p["kernel_id"] and kept["splits"] == p["splits"] for p in listed), (kept, listed)
+        tuned_bits = _to_bits(C)
+        res = oracle.check(tuned_bits, oracle.hgemm(A, B), K)
+        assert res["ok"] and res["non_finite"] == 0, res
+        again = torch.full((M, N), float("nan"), dtype=torch.float16, device=gpu)
+        print(f"[gpu] hgemm_auto (tuned) M={M} N={N} K={K}", flush=True)
+        hgemm_lib.call("hgemm_auto", Ad, Bd, again, M, N, K)
+        assert np.array_equal(_to_bits(again), tuned_bits)
+    finally:
+        hgemm_lib.forget_tuning()
+    assert not hgemm_lib.plan_is_tuned(M, N, K) and hgemm_lib.auto_plan(M, N, K) == model_plan

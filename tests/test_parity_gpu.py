@@ -505,8 +505,9 @@ def test_one_tile_row_in_k_slices(oracle, hgemm_lib, gpu, shape, slices):
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
-@pytest.mark.parametrize("shape,tail", [((103, 34304, 6656), (12, 16)), ((117, 39936, 1600), (56, 4)), ((50, 33024, 2048), (2, 6)),
-                                        ((128, 65792, 2112), (2, 6)), ((64, 32776, 4096), (1, 12)), ((76, 39552, 640), (0, 1))])
+@pytest.mark.parametrize("shape,tail", [((103, 34304, 6656), (12, 16)), ((117, 39936, 3200), (56, 4)), ((50, 33024, 4160), (2, 13)),
+                                        ((128, 65792, 4160), (2, 13)), ((64, 32776, 4096), (1, 12)), ((76, 39552, 640), (0, 1)),
+                                        ((60, 42496, 1536), (0, 1))])
 def test_one_tile_row_with_more_tiles_than_cus(oracle, hgemm_lib, gpu, shape, tail):
     """One row of 128x128 or 64x128 tiles against more column tiles than the chip has CUs: whole rounds in one launch
     (B copied non-temporally), the tiles beyond them in K slices that fill the chip, slices that differ by a chunk
