@@ -137,8 +137,8 @@ int hgemm_auto_plan_chained(size_t M, size_t N, size_t K);
 const char *hgemm_kernel_name(int kernel);
 /* Tuning on the caller's operands, for callers who run a shape many times: times up to max_plans (at most 12)
  * plans for the shape -- the one hgemm_auto would run, then the cost model's next best, each different in tile,
- * K slices or, for M <= 128, kernel -- with one untimed and three timed launches each (`flags`: 0 or
- * HGEMM_TUNE_COLD), and keeps the fastest for
+ * K slices or, for M <= 128, kernel -- with three untimed and 5 ... 40 timed launches each (`flags`: 0 or
+ * HGEMM_TUNE_COLD), and keeps the fastest (the model's own plan unless another is more than 3 % faster) for
  * every later hgemm_auto call of this shape in this process, from any thread; the hgemm_auto_plan* queries then
  * report the kept plan.  Blocks until the device is idle; C holds the product as the kept plan computes it (every
  * plan computes the same product; plans that slice K differently differ in the last bit of some outputs).  May
