@@ -306,3 +306,19 @@ def test_driver_flag_parser():
     assert r.returncode == 1 and "unknown flag -no_such_flag" in r.stderr
     r = subprocess.run([exe, "-M=abc"], capture_output=True, text=True, timeout=60)
     assert r.returncode == 1 and "is not a count" in r.stderr
+
+
+def test_plans_the_tuner_would_time(hgemm_lib):
+    """hgemm_auto_tune_plans (no launch): the first plan is hgemm_auto's own, no two are the same choice of kernel
+    and K slices unless they differ in how the last round of a large grid is run, small-M shapes offer the other
+    kernels of the rule table, and a shape with one possible kernel offers one plan."""
+    for shape in ((8192, 8192, 8192), (384, 6144, 5120), (64, 4096, 4096), (16, 28672, 4096), (1, 4096, 4096), (2048, 2048, 2048)):
+        plans = hgemm_lib.tune_plans(*shape, 8)
+        own = hgemm_lib.auto_plan(*shape)
+        assert 2 <= len(plans) <= 8 and (plans[0]["kernel_id"], plans[0]["splits"]) == (own["kernel_id"], own["splits"]), (shape, plans)
+    small = hgemm_lib.tune_plans(64, 4096, 4096, 8)
+    assert len({p["kernel"].split(",")[0] for p in small}) >= 3, small       # other kernels, not only other slice counts
+    assert len(hgemm_lib.tune_plans(100, 100, 100, 8)) == 1                  # the guarded kernel only
+    assert len(hgemm_lib.tune_plans(4095, 4095, 4095, 8)) == 1               # padded copies: the inner plan is not tuned
+    assert len(hgemm_lib.tune_plans(8192, 8192, 8192, 1)) == 1 and len(hgemm_lib.tune_plans(8192, 8192, 8192, 100)) <= 12
+    assert not hgemm_lib.plan_is_tuned(8192, 8192, 8192)
