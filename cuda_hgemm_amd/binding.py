@@ -50,7 +50,7 @@ HELPER_SYMBOLS = [
     "hgemm_tflops", "hgemm_bytes", "hgemm_version",
     "hgemm_reserve_workspace", "hgemm_release_workspace", "hgemm_auto_workspace_bytes",
     "hgemm_auto_static_workspace", "hgemm_static_workspace_bytes",
-    "hgemm_auto_tune", "hgemm_auto_tune_plans", "hgemm_auto_forget_tuning", "hgemm_auto_plan_is_tuned",
+    "hgemm_auto_tune", "hgemm_auto_tune_plans", "hgemm_auto_tune_result", "hgemm_auto_forget_tuning", "hgemm_auto_plan_is_tuned",
 ]
 
 
@@ -120,6 +120,8 @@ class HgemmLibrary:
         d.hgemm_auto_tune.restype = C.c_int
         d.hgemm_auto_tune_plans.argtypes = [_SZ, _SZ, _SZ, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         d.hgemm_auto_tune_plans.restype = C.c_int
+        d.hgemm_auto_tune_result.argtypes = [C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_float), C.POINTER(C.c_int)]
+        d.hgemm_auto_tune_result.restype = C.c_int
         d.hgemm_auto_forget_tuning.argtypes, d.hgemm_auto_forget_tuning.restype = [], None
         d.hgemm_auto_plan_is_tuned.argtypes, d.hgemm_auto_plan_is_tuned.restype = [_SZ, _SZ, _SZ], C.c_int
         d.hgemm_small_m_rule.argtypes = [C.c_int, C.POINTER(_SZ), C.POINTER(C.c_int)]
@@ -191,6 +193,16 @@ class HgemmLibrary:
         n = self.dll.hgemm_auto_tune_plans(M, N, K, max_plans, kernels, splits)
         return [{"kernel_id": kernels[i], "kernel": self.dll.hgemm_kernel_name(kernels[i]).decode(), "splits": splits[i]}
                 for i in range(n)]
+
+    def tune_results(self) -> List[dict]:
+        """What this thread's last ``tune`` measured, plan by plan in the order they were timed."""
+        out, i = [], 0
+        kernel, splits, ms, kept = C.c_int(0), C.c_int(0), C.c_float(0.0), C.c_int(0)
+        while self.dll.hgemm_auto_tune_result(i, C.byref(kernel), C.byref(splits), C.byref(ms), C.byref(kept)):
+            out.append({"kernel_id": kernel.value, "kernel": self.dll.hgemm_kernel_name(kernel.value).decode(),
+                        "splits": splits.value, "ms": ms.value, "kept": bool(kept.value)})
+            i += 1
+        return out
 
     def forget_tuning(self) -> None:
         self.dll.hgemm_auto_forget_tuning()

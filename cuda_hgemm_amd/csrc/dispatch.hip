@@ -587,6 +587,10 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
                 const size_t wgs = (M / c.bm) * (N / c.bn) * (size_t)s;
                 if (wgs > cus * (size_t)c.per_cu) break;
                 if (c.per_cu == 2 && (wgs <= cus || s > 1 || K / 64 >= W4_DEEP_MIN_CHUNKS)) break;
+                // most CUs busy and a long walk per workgroup: the 128x128 tile in K slices moves half the bytes per
+                // flop into LDS and is ahead (1024^2 x 7168: 25.3 us here, 22.2 us in four slices of 128x128 tiles;
+                // level at K = 5120, behind at 4096)
+                if (wgs * 4 > cus * 3 && shortest_slice(K, 64, s) >= 64 * 96) continue;
             }
             if (c.kernel == KERNEL_MID128_S2 && (s > 1 || K > 256)) break;
             // whole 64x64 tiles, at most one workgroup per CU: the four-wave tile is ahead of the one-wave tile on
@@ -920,6 +924,14 @@ extern "C" int hgemm_auto_tune_plans(size_t M, size_t N, size_t K, int max_plans
     return count;
 }
 
+// What the calling thread's last hgemm_auto_tune measured, plan by plan in the order they were timed.
+struct TuneRecord {
+    Plan plan;
+    float ms;
+};
+thread_local TuneRecord t_tune_records[TUNE_MOST_PLANS];
+thread_local int t_tune_record_count = 0, t_tune_kept = -1;
+
 // Streams over a buffer larger than the caches hold, so that what was cached before is not afterwards.
 __global__ void __launch_bounds__(256) cache_flush_kernel(floatx4 *buffer, size_t count, float value) {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -933,7 +945,8 @@ __global__ void __launch_bounds__(256) cache_flush_kernel(floatx4 *buffer, size_
 // plan three untimed launches, then 5 ... 40 timed ones (about half a millisecond of work) enqueued back to back, each
 // between events of its own on the null stream; with HGEMM_TUNE_COLD 512 MiB are streamed through the device before
 // each of them, so that A and B come from HBM as they do for a caller whose weights do not stay cached between
-// calls.  Another plan replaces the model's only if it is more than 3 % faster.  The call returns when the device is
+// calls.  About 30 ms of untimed work come first, so that every plan meets a settled clock.  Another plan replaces
+// the model's only if it is more than 3 % faster than the better of two timings of the model's.  The call returns when the device is
 // idle and C holds the product as the kept plan computes it.
 extern "C" int hgemm_auto_tune(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K,
                                int max_plans, int flags) {
@@ -982,6 +995,15 @@ extern "C" int hgemm_auto_tune(const hgemm_half *A, const hgemm_half *B, hgemm_h
     };
     int best = -1, timed = 0;
     float best_ms = 0.0f, first_ms = 0.0f;
+    t_tune_record_count = 0;
+    // The part is power-managed and takes tens of milliseconds of work to settle from idle: whoever is timed first is
+    // timed on a different clock (the model's own plan measured 13-23 % slower than the same kernel a moment later).
+    // So the device is kept busy with the first plan for about 30 ms before anything is timed, and that plan is timed
+    // once more after all the others; the better of its two timings counts.
+    if (count > 0 && run(plans[0])) {
+        float spent_ms = 0.0f;
+        for (int round = 0; round < 20 && spent_ms < 30.0f; ++round) spent_ms += 5.0f * time_plan(plans[0], 5);
+    }
     for (int i = 0; i < count; ++i) {
         if (!run(plans[i])) continue;
         // two untimed launches that also say how many timed ones make about half a millisecond of work (5 ... 40)
@@ -990,9 +1012,18 @@ extern "C" int hgemm_auto_tune(const hgemm_half *A, const hgemm_half *B, hgemm_h
         launches = launches < 5 ? 5 : launches > MOST_LAUNCHES ? MOST_LAUNCHES : launches;
         const float ms = time_plan(plans[i], launches);
         ++timed;
+        t_tune_records[t_tune_record_count++] = TuneRecord{plans[i], ms};
         if (i == 0) first_ms = ms;
         // the model's own plan stays unless another is ahead by more than the 3 % that two timings of one plan differ by
-        if (best < 0 || ms < (best == 0 ? 0.97f * first_ms : best_ms)) best = i, best_ms = ms;
+        if (best < 0 || ms < (best == 0 ? 0.97f * first_ms : best_ms)) best = i, best_ms = ms, t_tune_kept = t_tune_record_count - 1;
+    }
+    if (best > 0 && t_tune_record_count > 0 && same_choice(t_tune_records[0].plan, plans[0])) {
+        const float rough_ms = time_plan(plans[0], 2);
+        int launches = rough_ms > 0.0f ? (int)(0.5f / rough_ms) : MOST_LAUNCHES;
+        launches = launches < 5 ? 5 : launches > MOST_LAUNCHES ? MOST_LAUNCHES : launches;
+        const float again_ms = time_plan(plans[0], launches);
+        if (again_ms < t_tune_records[0].ms) t_tune_records[0].ms = again_ms;
+        if (best_ms >= 0.97f * t_tune_records[0].ms) best = 0, best_ms = t_tune_records[0].ms, t_tune_kept = 0;
     }
     for (int i = 0; i < MOST_LAUNCHES; ++i) {
         HGEMM_CHECK_HIP_ERROR(hipEventDestroy(start[i]));
@@ -1008,6 +1039,17 @@ extern "C" int hgemm_auto_tune(const hgemm_half *A, const hgemm_half *B, hgemm_h
     HGEMM_CHECK_HIP_ERROR(hipDeviceSynchronize());
     if (flush) HGEMM_CHECK_HIP_ERROR(hipFree(flush));
     return timed;
+}
+
+// The calling thread's last hgemm_auto_tune, plan by plan in the order they were timed: kernel id, K slices,
+// milliseconds per launch, whether it is the one that was kept.  Returns 0 past the last plan, else 1.
+extern "C" int hgemm_auto_tune_result(int index, int *kernel, int *splits, float *ms, int *kept) {
+    if (index < 0 || index >= t_tune_record_count) return 0;
+    if (kernel) *kernel = t_tune_records[index].plan.kernel;
+    if (splits) *splits = t_tune_records[index].plan.splits;
+    if (ms) *ms = t_tune_records[index].ms;
+    if (kept) *kept = index == t_tune_kept ? 1 : 0;
+    return 1;
 }
 
 // Forgets every tuned plan: hgemm_auto goes by the model again.

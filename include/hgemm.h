@@ -152,6 +152,9 @@ int hgemm_auto_tune(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, siz
 /* The plans hgemm_auto_tune would time, best first by the model, without a launch: kernel ids (for
  * hgemm_kernel_name) and K slices into arrays of max_plans entries (either may be NULL); returns their number. */
 int hgemm_auto_tune_plans(size_t M, size_t N, size_t K, int max_plans, int *kernels, int *splits);
+/* What the calling thread's last hgemm_auto_tune measured, plan by plan in the order they were timed: kernel id,
+ * K slices, milliseconds per launch, and whether that plan was the one kept.  Returns 0 past the last plan, else 1. */
+int hgemm_auto_tune_result(int index, int *kernel, int *splits, float *ms, int *kept);
 /* Forgets every kept plan; 1 if the shape has one. */
 void hgemm_auto_forget_tuning(void);
 int hgemm_auto_plan_is_tuned(size_t M, size_t N, size_t K);

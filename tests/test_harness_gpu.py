@@ -163,7 +163,10 @@ def test_tuning_on_the_callers_operands(oracle, hgemm_lib, gpu, shape):
         assert 1 <= timed <= len(listed) and hgemm_lib.plan_is_tuned(M, N, K)
         if shape == (100, 100, 100):
             assert timed == 1
+        results = hgemm_lib.tune_results()
+        assert len(results) == timed and sum(r["kept"] for r in results) == 1 and all(r["ms"] > 0 for r in results), results
         kept = hgemm_lib.auto_plan(M, N, K)
+        assert [r for r in results if r["kept"]][0]["kernel_id"] == kept["kernel_id"]
         assert any(kept["kernel_id"] == p["kernel_id"] and kept["splits"] == p["splits"] for p in listed), (kept, listed)
         tuned_bits = _to_bits(C)
         res = oracle.check(tuned_bits, oracle.hgemm(A, B), K)
