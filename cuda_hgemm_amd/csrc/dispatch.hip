@@ -932,18 +932,23 @@ struct TuneRecord {
 thread_local TuneRecord t_tune_records[TUNE_MOST_PLANS];
 thread_local int t_tune_record_count = 0, t_tune_kept = -1;
 
-// Streams over a buffer larger than the caches hold, so that what was cached before is not afterwards.
-__global__ void __launch_bounds__(256) cache_flush_kernel(floatx4 *buffer, size_t count, float value) {
+// Reads a buffer larger than the caches hold, so that what was cached before is not afterwards.  Reads, not writes:
+// the caches are left full of clean lines, as they are in a caller's loop over read-only weights; after a flush that
+// writes, the next kernel's loads must first push out dirty lines, which penalises kernels by how they load (the
+// streaming decode kernel read 30 us after a writing flush where it takes 13.5 us between other GEMMs).
+// `never` is a value no sum of the zero-filled buffer takes, so nothing is stored.
+__global__ void __launch_bounds__(256) cache_flush_kernel(floatx4 *buffer, size_t count, float never) {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride)
-        buffer[i] = floatx4{value, value, value, value};
+    floatx4 sum = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) sum += buffer[i];
+    if (sum[0] + sum[1] + sum[2] + sum[3] == never) buffer[0] = sum;
 }
 
 // Times the model's best plans for this shape on the caller's operands and keeps the fastest for every later
 // hgemm_auto call of the shape in this process: the first plan is the one hgemm_auto would run anyway, each next
 // one the best that is none of the earlier (another tile, another slice count, for M <= 128 another kernel).  Per
 // plan three untimed launches, then 5 ... 40 timed ones (about half a millisecond of work) enqueued back to back, each
-// between events of its own on the null stream; with HGEMM_TUNE_COLD 512 MiB are streamed through the device before
+// between events of its own on the null stream; with HGEMM_TUNE_COLD 512 MiB are read through the device before
 // each of them, so that A and B come from HBM as they do for a caller whose weights do not stay cached between
 // calls.  About 30 ms of untimed work come first, so that every plan meets a settled clock.  Another plan replaces
 // the model's only if it is more than 3 % faster than the better of two timings of the model's.  The call returns when the device is
@@ -959,6 +964,7 @@ extern "C" int hgemm_auto_tune(const hgemm_half *A, const hgemm_half *B, hgemm_h
         (void)hipGetLastError();
         flush = nullptr;  // no memory for it: the plans are timed on whatever the caches hold
     }
+    if (flush) HGEMM_CHECK_HIP_ERROR(hipMemsetAsync(flush, 0, FLUSH_BYTES, nullptr));
     constexpr int MOST_LAUNCHES = 40;
     hipEvent_t start[MOST_LAUNCHES], stop[MOST_LAUNCHES];
     for (int i = 0; i < MOST_LAUNCHES; ++i) {
@@ -977,7 +983,7 @@ extern "C" int hgemm_auto_tune(const hgemm_half *A, const hgemm_half *B, hgemm_h
     auto time_plan = [&](const Plan &p, int launches) {
         for (int i = 0; i < launches; ++i) {
             if (flush) {
-                cache_flush_kernel<<<dim3(2048), dim3(256), 0, nullptr>>>(flush, FLUSH_BYTES / sizeof(floatx4), (float)i);
+                cache_flush_kernel<<<dim3(2048), dim3(256), 0, nullptr>>>(flush, FLUSH_BYTES / sizeof(floatx4), 1.0f);
                 HGEMM_CHECK_HIP_ERROR(hipGetLastError());
             }
             HGEMM_CHECK_HIP_ERROR(hipEventRecord(start[i], nullptr));

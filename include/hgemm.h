@@ -145,7 +145,7 @@ const char *hgemm_kernel_name(int kernel);
  * allocate the workspace.  Returns the number of plans timed.  The vendor comparator is tuned the same way at its
  * first call of a shape (include/hgemm_hipblaslt.h).  No counterpart in the reference, whose kernels are one per
  * entry point. */
-#define HGEMM_TUNE_COLD 1 /* flags: stream 512 MiB through the device before every timed launch, so that A and B come
+#define HGEMM_TUNE_COLD 1 /* flags: read 512 MiB through the device before every timed launch, so that A and B come
                            * from HBM -- for callers whose operands (weights) do not stay cached between calls */
 int hgemm_auto_tune(const hgemm_half *A, const hgemm_half *B, hgemm_half *C, size_t M, size_t N, size_t K,
                     int max_plans, int flags);
