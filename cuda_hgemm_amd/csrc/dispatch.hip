@@ -419,6 +419,11 @@ constexpr SmallMRule SMALL_M_RULES[] = {
     // 32768, M = 65 and 128: 3-50 % ahead of the split-K kernels (N = 28672, K = 4096, M = 128: 53.1 -> 48.6 us,
     // 62.6 % of 8 TB/s), K = 384 ... 768 x N = 28672, 57344: 1.11 ... 1.24x; at N = 16384 mixed (0.84 ... 1.14), below
     // it behind (0.76 ... 0.90).  From K = 320, the shortest K its five-stage ring takes.
+    // N = 32769 ... 49152 are 257 ... 384 column tiles of 128, i.e. a second round of workgroups on a part of the chip, but
+    // at most 256 tiles of 192: one row of the 192x192 tile (its rows beyond M idle, which an HBM-bound kernel can
+    // afford) is 1.11 ... 1.34x up to K = 4096 over N = 34816 ... 49152 (M = 100, N = 36864, K = 1024: 27.1 -> 22.5 us);
+    // at K = 8192, where the 128x128 tile finishes its second round in K slices, 0.94 ... 1.03x.
+    {65, 128, 32769, 49152, 192, 6144, 0, ANY, 0, KERNEL_T192},
     {65, 128, 18432, ANY, 320, ANY, 0, ANY, 0, KERNEL_MID128},
     // M = 33 ... 64 there: the same kernel on a 64x128 tile, four waves side by side.  K = 384 ... 8192 x N = 18432 ...
     // 57344: 1-4 % ahead of the split-K 64x128 kernel where that ran unsliced (N = 28672, K = 4096, M = 64: 43.3 ->
@@ -432,7 +437,8 @@ constexpr SmallMRule SMALL_M_RULES[] = {
     // non-temporal too), the slice count by the split-K family's model: over N = 6144 ... 16384, M = 64 and 128,
     // K = 8192 and 16384: 0.99 ... 1.34x of the split-K kernels at their best slice count (median 1.17x; M = 128,
     // N = 10240, K = 16384: 106.9 -> 79.8 us); at K = 4096 mixed (0.92 ... 1.13x), at K = 2048 behind (0.80 ... 1.07x).
-    {65, 128, 6144, ANY, 8192, ANY, 0, ANY, 0, KERNEL_MID128},
+    // M = 65 ... 128 already from K = 6144: 1.01 ... 1.30x over N = 6144 ... 14336 at K = 6144 and 7168 (median 1.12x).
+    {65, 128, 6144, ANY, 6144, ANY, 0, ANY, 0, KERNEL_MID128},
     {33, 64, 6144, ANY, 8192, ANY, 0, ANY, 0, KERNEL_ROW64x128},
     // --- everything else with N % 64 == 0 and K % 64 == 0: the split-K family, the tile by M; 128-wide tiles where
     // N gives enough of them and is a multiple of 128 (they stream B better).
@@ -462,6 +468,7 @@ bool small_m_kernel_supports(int kernel, size_t M, size_t N, size_t K) {
         case KERNEL_DECODE_BN16: return decode_supports(M, N, K);
         case KERNEL_MID128:
         case KERNEL_ROW64x128: return N % 8 == 0 && K % 64 == 0 && K >= 64 * 5;
+        case KERNEL_T192: return N % 8 == 0 && K % 64 == 0 && K >= 64 * 3;
         case KERNEL_SPLIT_64x128:
         case KERNEL_SPLIT_128x128: return skinny_supports(M, N, K) && N % 128 == 0;
         default: return skinny_supports(M, N, K);
@@ -538,14 +545,15 @@ Plan plan_for(size_t M, size_t N, size_t K, const PlanLimits &limits) {
                 p.splits = waves;
                 break;
             }
+            case KERNEL_T192: p.splits = 1; break;
             case KERNEL_MID128:
             case KERNEL_ROW64x128: {
                 // up to one workgroup per CU: K slices by the split-K family's model (the same balance against the
                 // same partial sums); more tiles than CUs: whole rounds unsliced, the rest in K slices
                 const size_t tiles = div_ceil(N, (size_t)128);
-                // (from K = 8192: below, slices were measured level or behind -- M = 96, N = 18432, K = 4096: 40.8 us
-                // unsliced, 43.6 in three)
-                p.splits = tiles <= cus && K >= 8192 ? choose_splits(tiles, M, N, cus, K, slice_bytes, limits.partial_bytes, 5) : 1;
+                // (from K = 6144: below, slices were measured level or behind -- M = 96, N = 18432, K = 4096: 40.8 us
+                // unsliced, 43.6 in three; at K = 6144 and 7168 against N = 18432 1.00 ... 1.04x)
+                p.splits = tiles <= cus && K >= 6144 ? choose_splits(tiles, M, N, cus, K, slice_bytes, limits.partial_bytes, 5) : 1;
                 if (p.splits > 1) p.partial_bytes = (size_t)p.splits * slice_bytes;
                 if (tiles > cus) one_row_tail(p, r.kernel == KERNEL_MID128 ? 128 : 64, 5, N, K, cus, limits.partial_bytes);
                 break;

@@ -147,6 +147,8 @@ def test_small_m_rule_table(hgemm_lib):
             return M <= 32 and N % 32 == 0 and K % 256 == 0
         if kernel.startswith(("pipelined 128x128", "pipelined 64x128")):
             return N % 8 == 0 and K % 64 == 0 and K >= 320
+        if kernel.startswith("pipelined 192x192"):
+            return N % 8 == 0 and K % 64 == 0 and K >= 192
         if kernel.startswith("split-K"):
             wide = kernel.split()[1].split("x")[1] == "128"       # "split-K <BM>x<BN>x64, ...": 128-column tiles
             return N % 64 == 0 and K % 64 == 0 and (N % 128 == 0 or not wide)
@@ -166,7 +168,7 @@ def test_small_m_rule_table(hgemm_lib):
     family = lambda name: name.split(",")[0].replace("32 columns", "16 columns")   # the streaming kernel's two widths
     checked = 0
     for M in (1, 5, 6, 8, 9, 12, 13, 16, 17, 24, 25, 32, 33, 64, 65, 100, 128):    # both sides of every M class boundary
-        for N in (16, 48, 64, 272, 2048, 3072, 4096, 4112, 8192, 8208, 14336, 16384, 18432, 20488, 28672, 57344):
+        for N in (16, 48, 64, 272, 2048, 3072, 4096, 4112, 8192, 8208, 14336, 16384, 18432, 20488, 28672, 40960, 57344):
             for K in (64, 256, 384, 512, 1024, 1152, 2048, 2304, 4096, 4160, 6144, 8192, 12288, 16384, 32768):
                 expect = lookup(M, N, K)
                 if expect is None:

@@ -488,7 +488,8 @@ def test_one_tile_row_against_many_column_tiles(oracle, hgemm_lib, gpu, shape):
 
 
 @pytest.mark.parametrize("shape,slices", [((128, 6144, 8192), 5), ((64, 8192, 8192), 4), ((100, 12296, 8256), 5),
-                                           ((40, 18432, 12352), 7), ((32, 18432, 8192), 5), ((128, 16384, 8192), 2)])
+                                           ((40, 18432, 12352), 7), ((32, 18432, 8192), 5), ((128, 16384, 8192), 2),
+                                           ((100, 10240, 6144), 3), ((65, 6144, 7168), 5)])
 def test_one_tile_row_in_k_slices(oracle, hgemm_lib, gpu, shape, slices):
     """M = 17 ... 128 with a long K against fewer column tiles than CUs: the one-row 128x128 / 64x128 tiles with K in
     slices (B copied non-temporally in the sliced launch as well), slice counts that do and do not divide K's chunks,
@@ -505,8 +506,8 @@ def test_one_tile_row_in_k_slices(oracle, hgemm_lib, gpu, shape, slices):
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
-@pytest.mark.parametrize("shape,tail", [((103, 34304, 6656), (12, 16)), ((117, 39936, 3200), (56, 4)), ((50, 33024, 4160), (2, 13)),
-                                        ((128, 65792, 4160), (2, 13)), ((64, 32776, 4096), (1, 12)), ((76, 39552, 640), (0, 1)),
+@pytest.mark.parametrize("shape,tail", [((103, 34304, 6656), (12, 16)), ((117, 39936, 6464), (56, 4)), ((50, 33024, 4160), (2, 13)),
+                                        ((128, 65792, 4160), (2, 13)), ((64, 32776, 4096), (1, 12)), ((76, 52224, 640), (0, 1)),
                                         ((60, 42496, 1536), (0, 1))])
 def test_one_tile_row_with_more_tiles_than_cus(oracle, hgemm_lib, gpu, shape, tail):
     """One row of 128x128 or 64x128 tiles against more column tiles than the chip has CUs: whole rounds in one launch
@@ -523,6 +524,22 @@ def test_one_tile_row_with_more_tiles_than_cus(oracle, hgemm_lib, gpu, shape, ta
     _assert_close(oracle, first, oracle.hgemm(A, B), K)
     assert np.array_equal(first, second)
     At, Bt = oracle.fill((M, K), 44, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 44, 2, oracle.TERNARY, 0, 1)
+    assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
+
+
+@pytest.mark.parametrize("shape", [(100, 36864, 1024), (65, 34816, 512), (128, 49152, 2048), (96, 40968, 4096)])
+def test_one_row_of_192_wide_tiles(oracle, hgemm_lib, gpu, shape):
+    """M = 65 ... 128 against N = 32769 ... 49152: more than 256 column tiles of 128 but at most 256 of 192, so one row
+    of the 192x192 tile; rows of the tile beyond M, a last column tile that ends inside N."""
+    M, N, K = shape
+    plan = hgemm_lib.auto_plan(M, N, K)
+    assert plan["kernel"].startswith("pipelined 192x192x64") and plan["splits"] == 1 and plan["tail_tiles"] == 0, plan
+    A = oracle.fill((M, K), 49, 1, oracle.NORMAL, 0.0, 1.0)
+    B = oracle.fill((N, K), 49, 2, oracle.NORMAL, 0.0, 0.02)
+    first, second = _run(hgemm_lib, "hgemm_auto", A, B, gpu, repeat=2)
+    _assert_close(oracle, first, oracle.hgemm(A, B), K)
+    assert np.array_equal(first, second)
+    At, Bt = oracle.fill((M, K), 50, 1, oracle.TERNARY, 0, 1), oracle.fill((N, K), 50, 2, oracle.TERNARY, 0, 1)
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
