@@ -428,6 +428,9 @@ constexpr SmallMRule SMALL_M_RULES[] = {
     // M = 33 ... 64 there: the same kernel on a 64x128 tile, four waves side by side.  K = 384 ... 8192 x N = 18432 ...
     // 57344: 1-4 % ahead of the split-K 64x128 kernel where that ran unsliced (N = 28672, K = 4096, M = 64: 43.3 ->
     // 42.4 us, 70 % of 8 TB/s), 1.35x where it ran in two slices (N = 18432, 20480).
+    // (the 192-wide tile here only while the second round of 64x128 tiles would be almost empty: N = 34816: 0.97 ... 1.27x
+    // over K = 512 ... 4096; N = 40960: 0.91 ... 1.10x; N = 49152: 0.88 ... 1.03x)
+    {33, 64, 32769, 36864, 192, 6144, 0, ANY, 0, KERNEL_T192},
     {33, 64, 18432, ANY, 320, ANY, 0, ANY, 0, KERNEL_ROW64x128},
     // M = 17 ... 32 take that tile too once K is long (half its rows are idle, which an HBM-bound kernel can afford):
     // K = 4096, 8192 x N = 18432 ... 57344: 0.97 ... 1.27x over the split-K 32x64 kernel; at K <= 2048 that kernel stays

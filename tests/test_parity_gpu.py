@@ -506,8 +506,8 @@ def test_one_tile_row_in_k_slices(oracle, hgemm_lib, gpu, shape, slices):
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
-@pytest.mark.parametrize("shape,tail", [((103, 34304, 6656), (12, 16)), ((117, 39936, 6464), (56, 4)), ((50, 33024, 4160), (2, 13)),
-                                        ((128, 65792, 4160), (2, 13)), ((64, 32776, 4096), (1, 12)), ((76, 52224, 640), (0, 1)),
+@pytest.mark.parametrize("shape,tail", [((103, 34304, 6656), (12, 16)), ((117, 39936, 6464), (56, 4)), ((50, 33024, 6464), (2, 16)),
+                                        ((128, 65792, 4160), (2, 13)), ((64, 32776, 8192), (1, 16)), ((76, 52224, 640), (0, 1)),
                                         ((60, 42496, 1536), (0, 1))])
 def test_one_tile_row_with_more_tiles_than_cus(oracle, hgemm_lib, gpu, shape, tail):
     """One row of 128x128 or 64x128 tiles against more column tiles than the chip has CUs: whole rounds in one launch
@@ -527,10 +527,11 @@ def test_one_tile_row_with_more_tiles_than_cus(oracle, hgemm_lib, gpu, shape, ta
     assert np.array_equal(_run(hgemm_lib, "hgemm_auto", At, Bt, gpu), oracle.hgemm(At, Bt))
 
 
-@pytest.mark.parametrize("shape", [(100, 36864, 1024), (65, 34816, 512), (128, 49152, 2048), (96, 40968, 4096)])
+@pytest.mark.parametrize("shape", [(100, 36864, 1024), (65, 34816, 512), (128, 49152, 2048), (96, 40968, 4096),
+                                   (64, 34816, 4096), (40, 36864, 512)])
 def test_one_row_of_192_wide_tiles(oracle, hgemm_lib, gpu, shape):
-    """M = 65 ... 128 against N = 32769 ... 49152: more than 256 column tiles of 128 but at most 256 of 192, so one row
-    of the 192x192 tile; rows of the tile beyond M, a last column tile that ends inside N."""
+    """M = 65 ... 128 against N = 32769 ... 49152 (M = 33 ... 64: up to N = 36864): more than 256 column tiles of 128 but
+    at most 256 of 192, so one row of the 192x192 tile; rows of the tile beyond M, a last column tile that ends inside N."""
     M, N, K = shape
     plan = hgemm_lib.auto_plan(M, N, K)
     assert plan["kernel"].startswith("pipelined 192x192x64") and plan["splits"] == 1 and plan["tail_tiles"] == 0, plan
