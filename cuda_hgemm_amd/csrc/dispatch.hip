@@ -386,7 +386,9 @@ constexpr SmallMRule SMALL_M_RULES[] = {
     // K = 5120 1.07 ... 1.31x from N = 18432 (0.96 ... 1.08x at 14336), K = 8192 (ring kernel) 1.03 ... 1.14x, K = 4096
     // 1.04 ... 1.06x at M = 16 from N = 18432 (N = 28672: 40.1 -> 37.8 us) and level at M = 9, so from M = 13; M = 17 ... 24
     // (two row tiles, 64x128 pipelined tile before) 1.09 ... 1.13x at N = 18432 and 57344 and 0.93 ... 1.09x at N = 28672
-    // depending on the box; M = 32 and K <= 3072 mixed (0.68 ... 1.2x), so not taken.
+    // depending on the box; M = 25 ... 32 mixed up to N = 32000 (0.88 ... 1.07x) and 1.07 ... 1.24x against N = 40960 ...
+    // 151936 (the 64x128 tile's second and later rounds cost it more), so from N = 32768; K <= 3072 mixed (0.68 ... 1.2x),
+    // so not taken.
     {9, 16, 18432, ANY, 5120, 5120, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
     {9, 16, 14336, ANY, 10240, 10240, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
     {9, 16, 14336, ANY, 12288, 12288, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
@@ -394,6 +396,7 @@ constexpr SmallMRule SMALL_M_RULES[] = {
     {9, 16, 14336, ANY, 8192, 8192, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
     {13, 16, 18432, ANY, 4096, 4096, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
     {17, 24, 18432, ANY, 4096, 4096, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
+    {25, 32, 32768, ANY, 4096, 4096, (size_t)24 << 20, ANY, 0, KERNEL_DECODE_RESIDENT},
     // --- M = 9 ... 16: the ring kernel up to N = 8192 while K <= 4096 (K <= 8192 up to N = 4096); beyond, K slices
     // across workgroups are up to 29 % ahead -- except, with the non-temporal copies, against a B of 48 MB or more at
     // K = 2048, 4096 and 8192, where every wave walks 1024 of K (M = 12: 1.05 ... 1.29x, M = 16: 0.97 ... 1.23x over

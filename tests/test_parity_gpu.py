@@ -433,9 +433,9 @@ def test_decode_kernel_with_lds_rings(oracle, hgemm_lib, gpu, shape):
 
 
 @pytest.mark.parametrize("shape", [(16, 28672, 4096), (13, 18448, 4096), (9, 14336, 6144), (16, 14336, 8192), (11, 14352, 8192),
-                                   (17, 18432, 4096), (24, 20496, 4096), (20, 57344, 4096), (14, 16384, 6144)])
+                                   (17, 18432, 4096), (24, 20496, 4096), (20, 57344, 4096), (14, 16384, 6144), (32, 40976, 4096)])
 def test_decode_kernel_with_a_in_registers(oracle, hgemm_lib, gpu, shape):
-    """M = 9 ... 24 against N >= 14336: persistent workgroups that load their waves' K slices of A into registers once
+    """M = 9 ... 24 against N >= 14336 (up to M = 32 from N = 32768): persistent workgroups that load their waves' K slices of A into registers once
     and walk over 16-column tiles of C.  8, 12 and 16 chunks of K per wave, one and two row tiles of A, one and two
     workgroups per CU, tile counts that do and do not divide among the workgroups (some get one tile more; with 897
     tiles and 512 workgroups some get a single tile), rows of A beyond M."""
