@@ -324,3 +324,24 @@ def test_plans_the_tuner_would_time(hgemm_lib):
     assert len(hgemm_lib.tune_plans(4095, 4095, 4095, 8)) == 1               # padded copies: the inner plan is not tuned
     assert len(hgemm_lib.tune_plans(8192, 8192, 8192, 1)) == 1 and len(hgemm_lib.tune_plans(8192, 8192, 8192, 100)) <= 12
     assert not hgemm_lib.plan_is_tuned(8192, 8192, 8192)
+
+
+def test_slice_counts_of_the_split_k_family_on_timed_shapes(hgemm_lib):
+    """The model behind the split-K family's slice count against shapes that were timed at every count from 1 to 16
+    on an MI355X (microseconds at the count in brackets): the plan takes the fastest count, or one within 6 % of it."""
+    timed = {   # shape: (kernel, {slices: microseconds})
+        (96, 5120, 4096): ("split-K 128x64x64", {1: 27.6, 2: 19.6, 3: 16.3, 4: 22.3, 5: 20.4, 6: 19.8, 8: 23.8}),
+        (128, 13312, 4096): ("split-K 128x64x64", {1: 32.5, 2: 40.2, 3: 43.9, 4: 47.1, 6: 50.5, 8: 60.2}),
+        (48, 3072, 4096): ("split-K 64x64x64", {1: 21.2, 2: 14.5, 3: 12.2, 4: 10.7, 5: 10.3, 6: 12.5, 8: 12.5}),
+        (64, 4096, 4096): ("split-K 64x64x64", {1: 22.1, 2: 16.2, 3: 13.6, 4: 12.6, 5: 14.4, 6: 13.8, 8: 14.0}),
+        (128, 4096, 4096): ("split-K 128x64x64", {1: 28.8, 2: 20.2, 3: 16.9, 4: 15.9, 5: 21.4, 6: 20.7, 8: 20.8}),
+        (32, 4096, 4096): ("split-K 32x64x64", {1: 20.9, 2: 14.2, 3: 12.0, 4: 11.5, 5: 11.9, 6: 11.8, 8: 11.8}),
+        (96, 9216, 4096): ("split-K 128x64x64", {1: 29.1, 2: 35.1, 3: 28.2, 4: 33.0, 5: 31.1, 6: 35.0, 8: 38.5}),
+        (48, 13312, 2048): ("split-K 64x64x64", {1: 14.0, 2: 17.5, 3: 20.1, 4: 21.7, 5: 23.3, 6: 23.6, 8: 25.1}),
+        (22, 11264, 7296): ("split-K 32x64x64", {1: 36.5, 2: 36.5, 3: 36.7, 4: 33.1, 5: 33.8, 6: 35.4, 8: 35.6}),
+        (128, 9216, 2048): ("split-K 128x64x64", {1: 18.1, 2: 24.3, 3: 21.7, 4: 27.4, 5: 26.3, 6: 30.2, 8: 34.2}),
+    }
+    for shape, (kernel, us) in timed.items():
+        plan = hgemm_lib.auto_plan(*shape)
+        assert plan["kernel"].startswith(kernel) and plan["splits"] in us, (shape, plan)
+        assert us[plan["splits"]] <= 1.06 * min(us.values()), (shape, plan["splits"], us)
