@@ -436,9 +436,9 @@ constexpr SmallMRule SMALL_M_RULES[] = {
     {33, 64, 32769, 36864, 192, 6144, 0, ANY, 0, KERNEL_T192},
     {33, 64, 18432, ANY, 320, ANY, 0, ANY, 0, KERNEL_ROW64x128},
     // M = 17 ... 32 take that tile too once K is long (half its rows are idle, which an HBM-bound kernel can afford):
-    // K = 4096, 8192 x N = 18432 ... 57344: 0.97 ... 1.27x over the split-K 32x64 kernel; at K <= 2048 that kernel stays
-    // ahead against N >= 28672 (0.92 ... 0.98x).
-    {17, 32, 18432, ANY, 4096, ANY, 0, ANY, 0, KERNEL_ROW64x128},
+    // K = 4096, 8192 x N = 18432 ... 57344: 0.97 ... 1.27x over the split-K 32x64 kernel; K = 2944 ... 3584: 1.00 ... 1.15x;
+    // at K <= 2560 that kernel stays ahead or level against N >= 28672 (0.92 ... 1.05x).
+    {17, 32, 18432, ANY, 3072, ANY, 0, ANY, 0, KERNEL_ROW64x128},
     // M = 33 ... 128 against N = 6144 ... 18431 with a long K: the same two tiles with K in slices (their copies of B
     // non-temporal too), the slice count by the split-K family's model: over N = 6144 ... 16384, M = 64 and 128,
     // K = 8192 and 16384: 0.99 ... 1.34x of the split-K kernels at their best slice count (median 1.17x; M = 128,
