@@ -64,7 +64,9 @@ def _run(cmd):
 # kernel keeps its accumulators in AGPRs a0 ... a(4*TM*TN-1) that only its asm statements name:
 # it must use exactly that many AGPRs (one more would be an accumulator register the compiler
 # took for itself) and fewer than 256 VGPRs (beyond them the allocator starts looking for AGPRs).
-NO_SPILL_KERNELS = ("hgemm_pipelined_kernel", "hgemm_chained_kernel")
+# (the decode kernel that keeps A in registers is here because a spill of those registers would put A in scratch
+# memory and silently cost what the kernel exists to save)
+NO_SPILL_KERNELS = ("hgemm_pipelined_kernel", "hgemm_chained_kernel", "hgemm_decode_resident_kernel")
 # sources that must contain such kernels: a remark format the parser no longer understands
 # must not turn the guard into a no-op
 MUST_CHECK = {"dispatch.hip": NO_SPILL_KERNELS}

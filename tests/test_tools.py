@@ -108,25 +108,30 @@ def _remarks(kernels):
 
 
 def test_build_guard_for_the_inline_assembly_kernels():
-    """The build must fail when a hand-scheduled kernel spills, when a chained kernel's AGPR count is not exactly
-    its named accumulators (or its VGPRs reach 256), and when the guard finds nothing to check."""
+    """The build must fail when a hand-scheduled kernel (or the decode kernel that keeps A in registers) spills, when
+    a chained kernel's AGPR count is not exactly its named accumulators (or its VGPRs reach 256), and when the guard
+    finds nothing to check."""
     import pytest
     from cuda_hgemm_amd import build
     chained = "_ZN5hgemm20hgemm_chained_kernelINS_10PipeConfigILi256ELi256ELi64ELi2ELi2ELi2ELi16ELi1EEELb0ELb0EEEvPKDF16_"
     chained192 = "_ZN5hgemm20hgemm_chained_kernelINS_10PipeConfigILi192ELi192ELi64ELi2ELi2ELi3ELi16ELi0EEELb0ELb0EEEvPKDF16_"
     piped = "_ZN5hgemm22hgemm_pipelined_kernelINS_10PipeConfigILi128ELi128ELi64ELi2ELi2ELi5ELi16ELi0EEELb0ELb0EEEvPKDF16_"
+    resident = "_ZN5hgemm28hgemm_decode_resident_kernelILi1ELi16ELb1EEEvPKDF16_S2_PDF16_iiii"
     other = "_ZN5hgemm15pad_copy_kernelEPKDF16_PDF16_iiii"
     assert build._chained_accumulator_registers(chained) == 256
     assert build._chained_accumulator_registers(chained192) == 144
-    good = {chained: (179, 256, 0, 0), chained192: (139, 144, 0, 0), piped: (88, 64, 0, 0), other: (11, 0, 16, 2)}
-    assert build._check_no_spills("dispatch.hip", _remarks(good)) == {"hgemm_chained_kernel", "hgemm_pipelined_kernel"}
+    good = {chained: (179, 256, 0, 0), chained192: (139, 144, 0, 0), piped: (88, 64, 0, 0), resident: (160, 0, 0, 0),
+            other: (11, 0, 16, 2)}
+    assert build._check_no_spills("dispatch.hip", _remarks(good)) == {"hgemm_chained_kernel", "hgemm_pipelined_kernel",
+                                                                      "hgemm_decode_resident_kernel"}
     for bad in ({**good, piped: (88, 64, 8, 0)},             # scratch
                 {**good, chained: (179, 256, 0, 1)},         # a spilled VGPR
                 {**good, chained: (179, 260, 0, 0)},         # the compiler took AGPRs of its own
                 {**good, chained192: (139, 128, 0, 0)},      # fewer AGPRs than named accumulators
                 {**good, chained: (256, 256, 0, 0)},         # VGPRs exhausted
+                {**good, resident: (255, 0, 24, 6)},         # the rows of A it keeps in registers went to scratch
                 {other: (11, 0, 0, 0)},                      # nothing to check in a file that must have such kernels
-                {piped: (88, 64, 0, 0)}):                    # ... or only one of the two kinds
+                {piped: (88, 64, 0, 0)}):                    # ... or only one of the kinds
         with pytest.raises(RuntimeError):
             build._check_no_spills("dispatch.hip", _remarks(bad))
     with pytest.raises(RuntimeError):                        # a remark format the parser does not understand
